@@ -1,0 +1,172 @@
+/*
+ * llama3_host.h -- host-side interface of the MI355X LLaMA3 token loop.
+ *
+ * The functions and structs below keep the names, argument meaning and error
+ * behaviour (print a message, exit(1)) of the reference's host API, so that a
+ * caller written against the reference's headers links against this library
+ * unchanged.  Reference declarations replaced:
+ *   Tensor / Llama3Layer / Llama3          src/llama3/llama3.cuh:10-50
+ *   init_llama3, free_llama3, _free_tensor src/llama3/llama3.cuh:58-78
+ *   to_cuda                                src/llama3/llama3.cuh:80-90, llama3.cu:156-161
+ *   load_safetensor_weights                src/safetensor/safetensor.cuh:26-40, safetensor.cu:16-31
+ *   CudaCache, init_cache, inference       src/inference/inference.cuh:19-34,71, inference.cu:110-193
+ *   tokens_to_cuda                         src/tokenizer/tokenizer.cuh:66, tokenizer.cu:157-198
+ * Everything after "extensions" has no counterpart in the reference: a shape
+ * configuration (the reference hard-codes LLaMA3-8B in its kernels), the KV
+ * cache controls, greedy generation, seeded synthetic checkpoints and timing.
+ *
+ * The library is C-ABI throughout (extern "C", plain pointers and sizes).
+ */
+#ifndef LLAMA3_HOST_H
+#define LLAMA3_HOST_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef uint16_t llm_half; /* fp16 bit pattern (the reference's __half) */
+
+/* src/llama3/llama3.cuh:10-23 -- same fields, same order. */
+typedef struct {
+    int *ndim;
+    int *mem_len;
+    int *shape;
+    uint16_t *bf16_tensor;
+
+    int *d_ndim;
+    int *d_mem_len;
+    int *d_shape;
+    uint16_t *d_bf16_tensor;
+    llm_half *d_fp16_tensor;
+} Tensor;
+
+/* src/llama3/llama3.cuh:28-39 */
+typedef struct {
+    int layernum;
+    Tensor *input_layernorm;
+    Tensor *mlp_down_proj;
+    Tensor *mlp_gate_proj;
+    Tensor *mlp_up_proj;
+    Tensor *post_attention_layernorm;
+    Tensor *self_attn_k_proj;
+    Tensor *self_attn_o_proj;
+    Tensor *self_attn_q_proj;
+    Tensor *self_attn_v_proj;
+} Llama3Layer;
+
+/* src/llama3/llama3.cuh:44-50 (+ one trailing private field) */
+typedef struct {
+    Tensor *embed_tokens;
+    Tensor *lm_head;
+    Tensor *norm;
+    Llama3Layer **layers;
+    int n_layers;
+    void *device_slab; /* extension: the single HBM allocation that backs every weight */
+} Llama3;
+
+/* src/inference/inference.cuh:19-34 -- the reference's fields first, then the engine. */
+typedef struct {
+    Tensor *PN_X;
+    Tensor *Q;
+    Tensor *K;
+    Tensor *V;
+    float *d_attention_score_cache; /* always NULL: attention never materialises [H,T,T] */
+    llm_half *d_feedforward_cache_upgate;
+    llm_half *d_token_probdist; /* device fp16 logits of the last row */
+    llm_half *h_token_probdist;
+    float *f_token_probdist;
+    void *engine; /* extension: opaque engine state (KV cache, scratch, stream, graph) */
+} CudaCache;
+
+/* ---- reference API ---------------------------------------------------- */
+Llama3 *init_llama3(int n_layers);
+void free_llama3(Llama3 *llama3);
+void _free_tensor(Tensor *tensor);
+void load_safetensor_weights(Llama3 *llama3_model, const char *filename);
+void to_cuda(Llama3 *llama3);
+CudaCache *init_cache(Llama3 *llama3_model);
+int *tokens_to_cuda(int *tokens, int embed_size, Tensor *token_tensor);
+/* h_tokens[0] = n+1, ids in h_tokens[1..n]; returns the next token id. */
+int inference(Llama3 *llama3_model, Tensor *X, int *d_tokens, int *h_tokens, CudaCache *Cache);
+
+/* ---- extensions -------------------------------------------------------- */
+typedef struct {
+    int n_layers;
+    int d_model;
+    int n_heads;
+    int n_kv_heads;
+    int head_dim;
+    int ffn_dim;
+    int vocab;
+    int max_pos;
+    double rms_eps;
+    float rope_theta;
+} ModelConfig;
+
+/* LLaMA3-8B shapes with the reference's 2048-token limit. */
+ModelConfig llama3_config_8b(void);
+/* The CPU-runnable tiny model (2 layers, d 256, 8/2 heads, head_dim 32, FFN 768, vocab 4096). */
+ModelConfig llama3_config_tiny(void);
+
+/* init_cache with explicit shapes (init_cache() derives them from the tensor
+ * shapes, head_dim 128, max_pos 2048). */
+CudaCache *init_cache_cfg(Llama3 *llama3_model, const ModelConfig *cfg);
+void free_cache(CudaCache *Cache);
+
+/* KV-cached token loop.  prefill appends n tokens (any n >= 1) at the current
+ * position and returns the greedy next token; decode appends one. */
+int llama3_prefill(Llama3 *m, CudaCache *c, const int *tokens, int n);
+int llama3_decode(Llama3 *m, CudaCache *c, int token);
+void llama3_cache_reset(CudaCache *c);
+int llama3_cache_pos(const CudaCache *c);
+
+typedef struct {
+    double prefill_ms;     /* wall time of the prompt pass (HIP events) */
+    double decode_ms;      /* wall time of all decode steps */
+    int n_prompt;
+    int n_decode_steps;    /* steps timed in decode_ms */
+} GenStats;
+
+/* Greedy generation with the token id and position resident on the device:
+ * prompt pass, then n_decode-1 replays of one captured decode step.
+ * out_tokens receives n_decode ids (the first comes from the prompt pass). */
+int llama3_generate(Llama3 *m, CudaCache *c, const int *prompt, int n_prompt, int n_decode,
+                    int *out_tokens, GenStats *stats);
+
+/* Parity hooks: after the next prefill/decode call, hidden receives the
+ * residual stream after every layer for the rows of that call
+ * ([n_layers][n][d_model] fp16 bits, host memory); pass NULL to switch off.
+ * llama3_read_logits copies the fp16 logits of the last processed row. */
+void llama3_set_hidden_trace(CudaCache *c, llm_half *hidden);
+void llama3_read_logits(CudaCache *c, llm_half *logits);
+
+/* Choose between one hipGraph replay per decode step (1, default) and plain
+ * stream launches (0). */
+void llama3_set_use_graph(CudaCache *c, int on);
+
+/* Error hook.  Default prints the message and calls exit(1) as the reference
+ * does; tests install a handler that records instead. */
+typedef void (*llama3_error_fn)(const char *msg);
+void llama3_set_error_handler(llama3_error_fn fn);
+
+/* ---- seeded synthetic checkpoints -------------------------------------- */
+/* Counter-based generator: the value of element i of tensor id depends on
+ * (seed, id, i) only.  Matrices are N(0, 0.02) quantised through a 65536-level
+ * inverse-CDF table and rounded to bf16; RMSNorm gains are 1. */
+void seeded_normal_bf16(uint64_t seed, uint64_t tensor_id, size_t n, float sigma, uint16_t *out);
+void seeded_tokens(uint64_t seed, int n, int vocab, int *out);
+const uint16_t *seeded_unit_table_bf16(float sigma); /* 65536 entries */
+/* Fill every tensor of an init_llama3() model with host bf16 data of the
+ * shapes cfg implies (as load_safetensor_weights would leave it). */
+void seeded_fill_model(Llama3 *m, const ModelConfig *cfg, uint64_t seed);
+/* Write the same tensors as one safetensors file with HF LLaMA3 key names. */
+int seeded_write_safetensors(const ModelConfig *cfg, uint64_t seed, const char *path);
+uint64_t seeded_tensor_id(int layer, int slot);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,176 @@
+/*
+ * llmcu_hip.h -- thin C-ABI over the hand-written gfx950 (MI355X) kernels of
+ * the LLaMA3 token loop.  One entry point per kernel family; every pointer
+ * marked "device" is HBM memory, fp16 tensors are passed as uint16_t bit
+ * patterns, `stream` is a hipStream_t (NULL = the default stream).  All entry
+ * points return LLM_OK or an error code; llm_last_error() gives the text.
+ * Nothing here is asynchronous with respect to the given stream order.
+ *
+ * Each entry point names the launcher/kernel of the reference it replaces
+ * (paths under src/ of abhisheknair10/LLM.cu).  The host layer
+ * (llama3_host.h) is written against this header only and never includes the
+ * HIP runtime.
+ */
+#ifndef LLMCU_HIP_H
+#define LLMCU_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum {
+    LLM_OK = 0,
+    LLM_ERR_INVALID = 1, /* bad argument or a shape the kernels do not cover */
+    LLM_ERR_HIP = 2,     /* the HIP runtime reported an error */
+    LLM_ERR_NO_DEVICE = 3
+};
+
+typedef void *llm_stream_t;
+typedef void *llm_event_t;
+typedef void *llm_graph_t;
+
+/* ---- runtime (replaces the reference's direct cudart calls) ------------ */
+const char *llm_last_error(void);
+int llm_device_count(int *count);
+int llm_init(int device);                 /* select the device; fails unless it is gfx950 */
+int llm_device_name(char *buf, size_t n); /* e.g. "gfx950:sramecc+:xnack-" */
+int llm_device_cu_count(int *n);
+int llm_malloc(void **ptr, size_t bytes);           /* cudaMalloc   (inference.cu:101-108) */
+int llm_free(void *ptr);                            /* cudaFree */
+int llm_malloc_host(void **ptr, size_t bytes);      /* pinned host memory */
+int llm_free_host(void *ptr);
+int llm_memcpy_h2d(void *dst, const void *src, size_t bytes, llm_stream_t stream);
+int llm_memcpy_d2h(void *dst, const void *src, size_t bytes, llm_stream_t stream);
+int llm_memcpy_d2d(void *dst, const void *src, size_t bytes, llm_stream_t stream);
+int llm_fill_zero(void *dst, size_t bytes, llm_stream_t stream); /* a fill kernel, graph-safe */
+int llm_stream_create(llm_stream_t *stream);
+int llm_stream_destroy(llm_stream_t stream);
+int llm_stream_sync(llm_stream_t stream);
+int llm_device_sync(void);                          /* cudaDeviceSynchronize */
+int llm_event_create(llm_event_t *ev);
+int llm_event_destroy(llm_event_t ev);
+int llm_event_record(llm_event_t ev, llm_stream_t stream);
+int llm_event_sync(llm_event_t ev);
+int llm_event_elapsed_ms(llm_event_t start, llm_event_t stop, float *ms);
+int llm_graph_capture_begin(llm_stream_t stream);
+int llm_graph_capture_end(llm_stream_t stream, llm_graph_t *graph_exec);
+int llm_graph_launch(llm_graph_t graph_exec, llm_stream_t stream);
+int llm_graph_destroy(llm_graph_t graph_exec);
+
+/* ---- BF16 -> FP16 weight conversion ------------------------------------ */
+/* Replaces _kernel_wrapper_bf16_to_fp16 / _kernel_bf16_to_fp16
+ * (src/llama3/llama3.cu:219-254): dst[i] = fp16_rne(float(src[i] << 16)),
+ * NaN -> 0x7FFF.  Bit-exact.  4 algorithmic bytes per element. */
+int llm_bf16_to_fp16(const uint16_t *src_dev, uint16_t *dst_dev, size_t n, llm_stream_t stream);
+
+/* ---- embedding gather ---------------------------------------------------- */
+/* Replaces tokens_to_embeddings / kernel_tokens_to_embeddings
+ * (src/inference/inference.cu:196-223): out[t,:] = table[ids[t],:].
+ * ids are int32 on the device; an id outside [0, vocab) is rejected by
+ * writing a row of fp16 NaN (the reference reads out of bounds).
+ * ids_offset_dev (may be NULL): device int added to the index into ids_dev,
+ * so a captured graph can walk a token buffer. */
+int llm_embed_gather(const uint16_t *table_dev, const int32_t *ids_dev, const int32_t *ids_offset_dev,
+                     uint16_t *out_dev, int T, int d, int vocab, llm_stream_t stream);
+
+/* ---- RMSNorm --------------------------------------------------------------- */
+/* Replaces compute_layer_norm / kernel_compute_rms_norm
+ * (src/inference/inference.cu:282-363): y = fp16(x * g / sqrtf(eps + ss/d)),
+ * ss summed in the reference's own order (4-element partials, stride-halving
+ * tree), eps added in double as the reference's literal 1e-5 is.  y may alias
+ * x (the reference normalises in place).  Requires d % 4 == 0, d/4 a power of
+ * two, 64 <= d/4 <= 4096. */
+int llm_rmsnorm(const uint16_t *x_dev, const uint16_t *gain_dev, uint16_t *y_dev, int T, int d,
+                double eps, llm_stream_t stream);
+
+/* ---- residual add ---------------------------------------------------------- */
+/* Replaces add_norm / kernel_add_norm (src/inference/inference.cu:366-390):
+ * x = fp16(float(x) + float(res)). */
+int llm_add_residual(uint16_t *x_dev, const uint16_t *res_dev, size_t n, llm_stream_t stream);
+
+/* ---- RoPE -------------------------------------------------------------------- */
+/* Host helper: fills table[pos][i] = (cosf(a), sinf(a)), a = pos * 1/powf(theta, 2i/head_dim),
+ * i < head_dim/2, pos < max_pos, with the host libm -- the reference evaluates
+ * the same expression per element inside its kernel (inference.cu:673-678). */
+int llm_rope_table_host(float *table_host, int max_pos, int head_dim, float theta);
+/* Replaces rope_scaling / kernel_rope_scaling (src/inference/inference.cu:621-695):
+ * adjacent pairs (x[2p], x[2p+1]) of every head rotated in place by the
+ * angle of (pos0 + t, p % (head_dim/2)).  buf: [T, row_stride] fp16 with
+ * n_heads*head_dim leading columns used.  pos_dev (may be NULL): device int
+ * added to pos0, so a captured graph can advance without new arguments.
+ * table_dev: [max_pos][head_dim/2][2] floats from llm_rope_table_host. */
+int llm_rope(uint16_t *buf_dev, int T, int n_heads, int head_dim, int row_stride, int pos0,
+             const int32_t *pos_dev, const float *table_dev, int max_pos, llm_stream_t stream);
+/* Fused form used by the engine: rotates Q in place inside qkv ([T, (Hq+2Hkv)*hd]),
+ * rotates K and writes it into the K cache ([Hkv][max_pos][hd] per layer,
+ * rows pos0+t), and stores V into the V cache, which is kept transposed
+ * ([Hkv][hd][max_pos], columns pos0+t) so that P.V streams contiguous memory. */
+int llm_rope_kv_append(uint16_t *qkv_dev, uint16_t *k_cache_dev, uint16_t *v_cache_dev, int T,
+                       int n_heads, int n_kv_heads, int head_dim, int pos0, const int32_t *pos_dev,
+                       const float *table_dev, int max_pos, llm_stream_t stream);
+
+/* ---- projections -------------------------------------------------------------- */
+/* Replaces kernel_standard_tiled_gemm and its launchers compute_qkv_tensors,
+ * compute_output, the down projection of compute_feedforward
+ * (src/inference/inference.cu:393-449,561-618,967-976):
+ * out[t,n] = fp16(sum_k x[t,k] * w[n,k] (+ float(residual[t,n]))), fp32
+ * accumulation, w is [N,K] row-major.  With residual != NULL the result is
+ * fp16(fp16(sum) + residual), the reference's add_norm applied to the stored
+ * projection (inference.cu:377-390).  ldx/ldo/ldr are row strides in elements.
+ * T == 1 runs the bandwidth-bound GEMV, 2 <= T <= 16 the skinny kernel, larger
+ * T the MFMA GEMM.  K % 64 == 0 and N % 16 == 0 are required. */
+int llm_linear(const uint16_t *x_dev, int ldx, const uint16_t *w_dev, const uint16_t *residual_dev,
+               int ldr, uint16_t *out_dev, int ldo, int T, int N, int K, llm_stream_t stream);
+/* Replaces kernel_standard_tiled_gemm_ffn_swiglu (src/inference/inference.cu:455-519):
+ * out[t,n] = fp16(SiLU(sum_k x.wgate) * (sum_k x.wup)), neither sum rounded on its own. */
+int llm_linear_swiglu(const uint16_t *x_dev, int ldx, const uint16_t *wgate_dev,
+                      const uint16_t *wup_dev, uint16_t *out_dev, int ldo, int T, int N, int K,
+                      llm_stream_t stream);
+
+/* ---- attention ------------------------------------------------------------------ */
+/* Replaces compute_attention and its three kernels
+ * (src/inference/inference.cu:698-947) for one new row: causal GQA attention
+ * of the query at position ctx-1 over cache rows 0..ctx-1, kv_head = q_head /
+ * (Hq/Hkv), scores scaled by 1/sqrtf(head_dim), softmax and P.V in fp32.
+ * q: [Hq*hd] fp16; K cache [Hkv][max_pos][hd], V cache [Hkv][hd][max_pos];
+ * out: [Hq*hd] fp16.  ctx = ctx_host + (ctx_dev ? *ctx_dev : 0).
+ * max_pos % 64 == 0.  workspace: llm_attn_decode_workspace_bytes, zeroed once
+ * with llm_fill_zero before its first use (every call leaves it reusable);
+ * calls that share a workspace must not overlap. */
+size_t llm_attn_decode_workspace_bytes(int n_heads, int head_dim);
+int llm_attn_decode(const uint16_t *q_dev, const uint16_t *k_cache_dev, const uint16_t *v_cache_dev,
+                    uint16_t *out_dev, int ctx_host, const int32_t *ctx_dev, int n_heads,
+                    int n_kv_heads, int head_dim, int max_pos, void *workspace_dev,
+                    llm_stream_t stream);
+/* Same attention for T query rows at positions pos0..pos0+T-1 (prompt pass),
+ * streaming softmax on MFMA tiles; never materialises [H,T,T].
+ * q: [T, ldq] with head h at columns h*hd; out: [T, ldo].  Cache rows beyond
+ * the written positions must hold finite values (zero the caches once). */
+int llm_attn_prefill(const uint16_t *q_dev, int ldq, const uint16_t *k_cache_dev,
+                     const uint16_t *v_cache_dev, uint16_t *out_dev, int ldo, int T, int pos0,
+                     int n_heads, int n_kv_heads, int head_dim, int max_pos, llm_stream_t stream);
+
+/* ---- LM head + argmax ------------------------------------------------------------ */
+/* Replaces compute_lm_head (src/inference/inference.cu:1003-1028) with the
+ * north-star's greedy selection instead of the host sampler: logits =
+ * fp16(x . w^T) for one row, token = argmax over the fp16 logits, lowest index
+ * on ties, NaN never selected.  logits_dev: [vocab] fp16 (kept, as the
+ * reference keeps d_token_probdist).  token_dev: device int32 result.
+ * tokens_dev/pos_dev (may be NULL): when given, the token is also stored at
+ * tokens_dev[*pos_dev + 1] and *pos_dev is incremented, which lets a captured
+ * decode step feed the next one. */
+size_t llm_lmhead_workspace_bytes(int vocab);
+int llm_lmhead_argmax(const uint16_t *x_dev, const uint16_t *w_dev, uint16_t *logits_dev,
+                      int32_t *token_dev, int32_t *tokens_dev, int32_t *pos_dev, int vocab, int K,
+                      void *workspace_dev, llm_stream_t stream);
+/* argmax alone over fp16 values (same tie/NaN rule). */
+int llm_argmax_f16(const uint16_t *logits_dev, int n, int32_t *token_dev, void *workspace_dev,
+                   llm_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,90 @@
+// Shared device/host helpers for the gfx950 kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "llmcu_hip.h"
+
+typedef _Float16 half_t;
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef float float16_t __attribute__((ext_vector_type(16)));
+typedef uint32_t uint4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t uint2_t __attribute__((ext_vector_type(2)));
+
+#define WAVE 64
+
+// ---- error plumbing -------------------------------------------------------
+void llm_set_error(const char *fmt, ...) __attribute__((format(printf, 1, 2)));
+
+#define LLM_HIP_CHECK(expr)                                                          \
+    do {                                                                             \
+        hipError_t _e = (expr);                                                      \
+        if (_e != hipSuccess) {                                                      \
+            llm_set_error("%s: %s (%s:%d)", #expr, hipGetErrorString(_e), __FILE__, __LINE__); \
+            return LLM_ERR_HIP;                                                      \
+        }                                                                            \
+    } while (0)
+
+#define LLM_REQUIRE(cond, ...)            \
+    do {                                  \
+        if (!(cond)) {                    \
+            llm_set_error(__VA_ARGS__);   \
+            return LLM_ERR_INVALID;       \
+        }                                 \
+    } while (0)
+
+// Launch check: hipGetLastError right after the <<<>>>.
+#define LLM_LAUNCH_CHECK(name)                                                      \
+    do {                                                                            \
+        hipError_t _e = hipGetLastError();                                          \
+        if (_e != hipSuccess) {                                                     \
+            llm_set_error("launch of %s: %s", name, hipGetErrorString(_e));         \
+            return LLM_ERR_HIP;                                                     \
+        }                                                                           \
+    } while (0)
+
+static inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// ---- device helpers ---------------------------------------------------------
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off);
+    return v;
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) v = fmaxf(v, __shfl_xor(v, off));
+    return v;
+}
+
+// 8 fp16 x 8 fp16 -> fp32, accumulated with v_dot2_f32_f16.
+__device__ __forceinline__ float dot8(half8_t a, half8_t b, float acc) {
+    acc = __builtin_amdgcn_fdot2(half2_t{a[0], a[1]}, half2_t{b[0], b[1]}, acc, false);
+    acc = __builtin_amdgcn_fdot2(half2_t{a[2], a[3]}, half2_t{b[2], b[3]}, acc, false);
+    acc = __builtin_amdgcn_fdot2(half2_t{a[4], a[5]}, half2_t{b[4], b[5]}, acc, false);
+    acc = __builtin_amdgcn_fdot2(half2_t{a[6], a[7]}, half2_t{b[6], b[7]}, acc, false);
+    return acc;
+}
+
+__device__ __forceinline__ half8_t load8(const half_t *p) { return *reinterpret_cast<const half8_t *>(p); }
+__device__ __forceinline__ void store8(half_t *p, half8_t v) { *reinterpret_cast<half8_t *>(p) = v; }
+
+// fp16 result with an optional residual: the reference stores the projection
+// as fp16 and then adds the fp16 residual in fp32 (two roundings).
+__device__ __forceinline__ half_t finish(float acc, const half_t *res) {
+    half_t h = (half_t)acc;
+    if (res) h = (half_t)((float)h + (float)*res);
+    return h;
+}
+
+// Bit pattern of the fp16 logit mapped to an unsigned key that orders like
+// the value (NaN excluded by the caller): used by the argmax reductions.
+__device__ __forceinline__ uint32_t f16_order_key(uint16_t bits) {
+    // -0 and +0 must compare equal: map -0 to +0 first.
+    if (bits == 0x8000u) bits = 0;
+    return (bits & 0x8000u) ? (uint32_t)(0x7fffu - (bits & 0x7fffu)) : (uint32_t)(0x8000u + bits);
+}

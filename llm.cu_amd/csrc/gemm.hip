@@ -1,0 +1,322 @@
+// Projections for more than one token: out = x . w^T with fp32 accumulation
+// on the MFMA units.  w is [N, K] row-major and x is [T, K] row-major, so both
+// MFMA operands are K-contiguous and every lane's fragment is one 16-byte load.
+//
+//  * skinny (2 <= T <= 16): one workgroup per 16 weight rows, its 8 wavefronts
+//    split K, v_mfma_f32_16x16x32_f16 with the token rows as the M side.
+//    HBM-bound: weights are read once, straight from global memory.
+//  * tiled GEMM (T > 16): BM x BN macro-tiles staged through LDS (double
+//    buffered, padded rows), v_mfma_f32_32x32x16_f16, wave tiles up to 128x128.
+//
+// MFMA operand layouts used below (wave64):
+//   16x16x32: A lane l -> row l%16, k = 8*(l/16)..+7;  B lane l -> col l%16, same k;
+//             D lane l -> col l%16, rows 4*(l/16)+i, i<4.
+//   32x32x16: A lane l -> row l%32, k = 8*(l/32)..+7;  B lane l -> col l%32, same k;
+//             D lane l -> col l%32, rows 8*(i/4) + 4*(l/32) + i%4, i<16.
+#include <cmath>
+
+#include "common.hpp"
+
+int gemv_launch(const half_t *x, const half_t *w, const half_t *res, half_t *out, int N, int K, hipStream_t s);
+int gemv_swiglu_launch(const half_t *x, const half_t *wg, const half_t *wu, half_t *out, int N, int K,
+                       hipStream_t s);
+
+__device__ __forceinline__ float silu_g(float g) { return g / (1.0f + expf(-g)); }
+
+// ---------------------------------------------------------------------------
+// skinny
+// ---------------------------------------------------------------------------
+#define SK_WAVES 8
+
+template <bool SWIGLU>
+__global__ __launch_bounds__(SK_WAVES * 64) void skinny_kernel(const half_t *__restrict__ x, int ldx,
+                                                               const half_t *__restrict__ w,
+                                                               const half_t *__restrict__ w2,
+                                                               const half_t *__restrict__ res, int ldr,
+                                                               half_t *__restrict__ out, int ldo, int T,
+                                                               int N, int K) {
+    __shared__ float red[SWIGLU ? 2 : 1][SK_WAVES][64][4];
+    const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
+    const int r = lane % 16, g = lane / 16;
+    const int n0 = blockIdx.x * 16;
+    const int nrow = n0 + r < N ? n0 + r : N - 1;
+    const int mrow = r < T ? r : T - 1;
+    const int kslice = K / SK_WAVES; // multiple of 32
+    const int kbeg = wave * kslice;
+    const half_t *xp = x + (size_t)mrow * ldx + kbeg + 8 * g;
+    const half_t *wp = w + (size_t)nrow * K + kbeg + 8 * g;
+    const half_t *wp2 = SWIGLU ? w2 + (size_t)nrow * K + kbeg + 8 * g : nullptr;
+    float4_t acc = {0.f, 0.f, 0.f, 0.f}, acc2 = {0.f, 0.f, 0.f, 0.f};
+    constexpr int U = 4;
+    int k = 0;
+    for (; k + 32 * U <= kslice; k += 32 * U) {
+        half8_t a[U], b[U], b2[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            b[u] = load8(wp + k + 32 * u);
+            if (SWIGLU) b2[u] = load8(wp2 + k + 32 * u);
+            a[u] = load8(xp + k + 32 * u);
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[u], b[u], acc, 0, 0, 0);
+            if (SWIGLU) acc2 = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[u], b2[u], acc2, 0, 0, 0);
+        }
+    }
+    for (; k < kslice; k += 32) {
+        half8_t a = load8(xp + k), b = load8(wp + k);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, acc, 0, 0, 0);
+        if (SWIGLU) acc2 = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, load8(wp2 + k), acc2, 0, 0, 0);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        red[0][wave][lane][i] = acc[i];
+        if (SWIGLU) red[SWIGLU ? 1 : 0][wave][lane][i] = acc2[i];
+    }
+    __syncthreads();
+    if (wave == 0) {
+        const int n = n0 + lane % 16;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int m = 4 * (lane / 16) + i;
+            float s = 0.f, s2 = 0.f;
+#pragma unroll
+            for (int wv = 0; wv < SK_WAVES; ++wv) {
+                s += red[0][wv][lane][i];
+                if (SWIGLU) s2 += red[SWIGLU ? 1 : 0][wv][lane][i];
+            }
+            if (m < T && n < N) {
+                if (SWIGLU) {
+                    out[(size_t)m * ldo + n] = (half_t)(silu_g(s) * s2);
+                } else {
+                    out[(size_t)m * ldo + n] = finish(s, res ? res + (size_t)m * ldr + n : nullptr);
+                }
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// tiled MFMA GEMM
+// ---------------------------------------------------------------------------
+#define GEMM_BK 64
+#define GEMM_PAD 8
+#define GEMM_LD (GEMM_BK + GEMM_PAD) // LDS row stride in halves: 144 B, so 8 rows hit 8 different 16-byte bank groups
+
+enum { EPI_PLAIN = 0, EPI_SWIGLU = 1 };
+
+// BM x BN macro-tile, WGM x WGN wavefronts, NB = number of weight matrices
+// (2 for the fused gate/up pair: BN rows of each).
+template <int BM, int BN, int WGM, int WGN, int NB>
+__global__ __launch_bounds__(WGM *WGN * 64) void gemm_kernel(const half_t *__restrict__ x, int ldx,
+                                                             const half_t *__restrict__ w,
+                                                             const half_t *__restrict__ w2,
+                                                             const half_t *__restrict__ res, int ldr,
+                                                             half_t *__restrict__ out, int ldo, int T,
+                                                             int N, int K, int tiles_m, int tiles_n) {
+    constexpr int THREADS = WGM * WGN * 64;
+    constexpr int TM = BM / WGM, TN = BN / WGN; // wave tile
+    constexpr int FM = TM / 32, FN = TN / 32;   // 32x32 fragments per wave
+    constexpr int A_LOADS = BM * GEMM_BK / 8 / THREADS;
+    constexpr int B_LOADS = BN * GEMM_BK / 8 / THREADS;
+    static_assert(A_LOADS >= 1 && B_LOADS >= 1, "tile too small for the workgroup");
+    static_assert(BM * GEMM_BK / 8 % THREADS == 0 && BN * GEMM_BK / 8 % THREADS == 0, "uneven staging");
+
+    extern __shared__ __attribute__((aligned(16))) half_t lds[];
+    half_t *As = lds;                                    // [2][BM][GEMM_LD]
+    half_t *Bs = lds + 2 * BM * GEMM_LD;                 // [2][NB][BN][GEMM_LD]
+
+    // XCD-aware tile order: consecutive workgroup ids land on different XCDs
+    // (8 of them), so give each XCD a contiguous run of tiles, and walk the
+    // tiles of a run down M first so neighbours share the weight (B) tile in
+    // that XCD's L2.
+    const int nblk = tiles_m * tiles_n;
+    int bid = blockIdx.x;
+    {
+        const int per = nblk / 8;
+        if (per > 0 && bid < per * 8) bid = (bid % 8) * per + bid / 8;
+    }
+    const int tm = bid % tiles_m, tn = bid / tiles_m;
+    const int m0 = tm * BM, n0 = tn * BN;
+
+    const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
+    const int wm = wave % WGM, wn = wave / WGM;
+
+    // staging map: 8 threads cover one 64-half row
+    const int srow = tid / 8, scol = (tid % 8) * 8;
+    constexpr int ROWS_PER_PASS = THREADS / 8;
+
+    const half_t *ag[A_LOADS];
+    const half_t *bg[NB][B_LOADS];
+#pragma unroll
+    for (int i = 0; i < A_LOADS; ++i) {
+        int row = m0 + srow + i * ROWS_PER_PASS;
+        row = row < T ? row : T - 1;
+        ag[i] = x + (size_t)row * ldx + scol;
+    }
+#pragma unroll
+    for (int i = 0; i < B_LOADS; ++i) {
+        int row = n0 + srow + i * ROWS_PER_PASS;
+        row = row < N ? row : N - 1;
+        bg[0][i] = w + (size_t)row * K + scol;
+        if (NB == 2) bg[NB - 1][i] = w2 + (size_t)row * K + scol;
+    }
+
+    float16_t acc[NB][FM][FN];
+#pragma unroll
+    for (int b = 0; b < NB; ++b)
+#pragma unroll
+        for (int i = 0; i < FM; ++i)
+#pragma unroll
+            for (int j = 0; j < FN; ++j)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) acc[b][i][j][e] = 0.f;
+
+    half8_t ra[A_LOADS], rb[NB][B_LOADS];
+    auto gload = [&](int k0) {
+#pragma unroll
+        for (int i = 0; i < A_LOADS; ++i) ra[i] = load8(ag[i] + k0);
+#pragma unroll
+        for (int b = 0; b < NB; ++b)
+#pragma unroll
+            for (int i = 0; i < B_LOADS; ++i) rb[b][i] = load8(bg[b][i] + k0);
+    };
+    auto sstore = [&](int buf) {
+        half_t *a = As + buf * BM * GEMM_LD;
+#pragma unroll
+        for (int i = 0; i < A_LOADS; ++i) store8(a + (srow + i * ROWS_PER_PASS) * GEMM_LD + scol, ra[i]);
+#pragma unroll
+        for (int b = 0; b < NB; ++b) {
+            half_t *bb = Bs + (buf * NB + b) * BN * GEMM_LD;
+#pragma unroll
+            for (int i = 0; i < B_LOADS; ++i) store8(bb + (srow + i * ROWS_PER_PASS) * GEMM_LD + scol, rb[b][i]);
+        }
+    };
+
+    const int nk = K / GEMM_BK;
+    gload(0);
+    sstore(0);
+    __syncthreads();
+
+    const int frow = lane % 32, fk = (lane / 32) * 8;
+    for (int kt = 0; kt < nk; ++kt) {
+        const int buf = kt & 1;
+        if (kt + 1 < nk) gload((kt + 1) * GEMM_BK);
+        const half_t *a = As + buf * BM * GEMM_LD + (wm * TM + frow) * GEMM_LD + fk;
+#pragma unroll
+        for (int ks = 0; ks < GEMM_BK / 16; ++ks) {
+            half8_t af[FM];
+#pragma unroll
+            for (int i = 0; i < FM; ++i) af[i] = load8(a + i * 32 * GEMM_LD + ks * 16);
+#pragma unroll
+            for (int b = 0; b < NB; ++b) {
+                const half_t *bp = Bs + (buf * NB + b) * BN * GEMM_LD + (wn * TN + frow) * GEMM_LD + fk;
+                half8_t bf[FN];
+#pragma unroll
+                for (int j = 0; j < FN; ++j) bf[j] = load8(bp + j * 32 * GEMM_LD + ks * 16);
+#pragma unroll
+                for (int i = 0; i < FM; ++i)
+#pragma unroll
+                    for (int j = 0; j < FN; ++j)
+                        acc[b][i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf[j], acc[b][i][j], 0, 0, 0);
+            }
+        }
+        if (kt + 1 < nk) sstore(buf ^ 1);
+        __syncthreads();
+    }
+
+    // epilogue: D lane l -> col l%32, rows 8*(e/4) + 4*(l/32) + e%4
+    const int ccol = lane % 32, crow0 = 4 * (lane / 32);
+#pragma unroll
+    for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int j = 0; j < FN; ++j) {
+            const int n = n0 + wn * TN + j * 32 + ccol;
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const int m = m0 + wm * TM + i * 32 + 8 * (e / 4) + crow0 + (e % 4);
+                if (m < T && n < N) {
+                    if (NB == 2) {
+                        out[(size_t)m * ldo + n] = (half_t)(silu_g(acc[0][i][j][e]) * acc[NB - 1][i][j][e]);
+                    } else {
+                        out[(size_t)m * ldo + n] = finish(acc[0][i][j][e], res ? res + (size_t)m * ldr + n : nullptr);
+                    }
+                }
+            }
+        }
+}
+
+template <int BM, int BN, int WGM, int WGN, int NB>
+static int gemm_launch(const half_t *x, int ldx, const half_t *w, const half_t *w2, const half_t *res, int ldr,
+                       half_t *out, int ldo, int T, int N, int K, hipStream_t s) {
+    const int tiles_m = (T + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
+    const size_t smem = sizeof(half_t) * (2 * (size_t)BM * GEMM_LD + 2 * (size_t)NB * BN * GEMM_LD);
+    auto kern = gemm_kernel<BM, BN, WGM, WGN, NB>;
+    static bool attr_set = false;
+    if (!attr_set && smem > 48 * 1024) {
+        LLM_HIP_CHECK(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+        attr_set = true;
+    }
+    kern<<<dim3(tiles_m * tiles_n), dim3(WGM * WGN * 64), smem, s>>>(x, ldx, w, w2, res, ldr, out, ldo, T, N, K,
+                                                                     tiles_m, tiles_n);
+    LLM_LAUNCH_CHECK("gemm_kernel");
+    return LLM_OK;
+}
+
+// ---------------------------------------------------------------------------
+static int check_linear(const void *x, int ldx, const void *w, const void *out, int ldo, int T, int N, int K,
+                        const char *who) {
+    LLM_REQUIRE(x && w && out, "%s: null pointer", who);
+    LLM_REQUIRE(T >= 0 && N > 0 && K > 0, "%s: T=%d N=%d K=%d", who, T, N, K);
+    LLM_REQUIRE(K % 64 == 0, "%s: K=%d must be a multiple of 64", who, K);
+    LLM_REQUIRE(N % 16 == 0, "%s: N=%d must be a multiple of 16", who, N);
+    LLM_REQUIRE(ldx >= K && ldx % 8 == 0 && ldo >= N, "%s: ldx=%d ldo=%d", who, ldx, ldo);
+    LLM_REQUIRE(aligned16(x) && aligned16(w), "%s: x and w must be 16-byte aligned", who);
+    return LLM_OK;
+}
+
+extern "C" {
+
+int llm_linear(const uint16_t *x, int ldx, const uint16_t *w, const uint16_t *residual, int ldr, uint16_t *out,
+               int ldo, int T, int N, int K, llm_stream_t stream) {
+    int rc = check_linear(x, ldx, w, out, ldo, T, N, K, "llm_linear");
+    if (rc != LLM_OK) return rc;
+    LLM_REQUIRE(!residual || ldr >= N, "llm_linear: ldr=%d", ldr);
+    if (T == 0) return LLM_OK;
+    hipStream_t s = (hipStream_t)stream;
+    const half_t *xp = (const half_t *)x, *wp = (const half_t *)w, *rp = (const half_t *)residual;
+    half_t *op = (half_t *)out;
+    if (T == 1) return gemv_launch(xp, wp, rp, op, N, K, s);
+    if (T <= 16 && K % (SK_WAVES * 32) == 0) {
+        skinny_kernel<false><<<dim3((N + 15) / 16), dim3(SK_WAVES * 64), 0, s>>>(xp, ldx, wp, nullptr, rp, ldr, op,
+                                                                               ldo, T, N, K);
+        LLM_LAUNCH_CHECK("skinny_kernel");
+        return LLM_OK;
+    }
+    if (T <= 64 || N < 256) return gemm_launch<64, 64, 2, 2, 1>(xp, ldx, wp, nullptr, rp, ldr, op, ldo, T, N, K, s);
+    if (T <= 128) return gemm_launch<128, 128, 2, 2, 1>(xp, ldx, wp, nullptr, rp, ldr, op, ldo, T, N, K, s);
+    return gemm_launch<256, 256, 2, 2, 1>(xp, ldx, wp, nullptr, rp, ldr, op, ldo, T, N, K, s);
+}
+
+int llm_linear_swiglu(const uint16_t *x, int ldx, const uint16_t *wgate, const uint16_t *wup, uint16_t *out,
+                      int ldo, int T, int N, int K, llm_stream_t stream) {
+    int rc = check_linear(x, ldx, wgate, out, ldo, T, N, K, "llm_linear_swiglu");
+    if (rc != LLM_OK) return rc;
+    LLM_REQUIRE(wup && aligned16(wup), "llm_linear_swiglu: wup");
+    if (T == 0) return LLM_OK;
+    hipStream_t s = (hipStream_t)stream;
+    const half_t *xp = (const half_t *)x, *gp = (const half_t *)wgate, *up = (const half_t *)wup;
+    half_t *op = (half_t *)out;
+    if (T == 1) return gemv_swiglu_launch(xp, gp, up, op, N, K, s);
+    if (T <= 16 && K % (SK_WAVES * 32) == 0) {
+        skinny_kernel<true><<<dim3((N + 15) / 16), dim3(SK_WAVES * 64), 0, s>>>(xp, ldx, gp, up, nullptr, 0, op, ldo,
+                                                                              T, N, K);
+        LLM_LAUNCH_CHECK("skinny_kernel<swiglu>");
+        return LLM_OK;
+    }
+    if (T <= 64 || N < 256) return gemm_launch<64, 64, 2, 2, 2>(xp, ldx, gp, up, nullptr, 0, op, ldo, T, N, K, s);
+    if (T <= 128) return gemm_launch<128, 64, 2, 2, 2>(xp, ldx, gp, up, nullptr, 0, op, ldo, T, N, K, s);
+    return gemm_launch<256, 128, 2, 2, 2>(xp, ldx, gp, up, nullptr, 0, op, ldo, T, N, K, s);
+}
+
+} // extern "C"

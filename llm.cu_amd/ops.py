@@ -1,0 +1,182 @@
+"""numpy-in / numpy-out wrappers of the kernel entry points (one C-ABI call
+each).  Arrays are uint16 fp16/bf16 bit patterns unless noted.  Used by the
+parity tests and the micro-benchmarks; the token loop itself lives in the C++
+host layer (engine.py binds it)."""
+import ctypes as C
+
+import numpy as np
+
+from . import capi
+from .capi import DevBuf, check, lib
+
+
+def _u16(a):
+    a = np.ascontiguousarray(a)
+    if a.dtype == np.float16:
+        a = a.view(np.uint16)
+    assert a.dtype == np.uint16, a.dtype
+    return a
+
+
+def bf16_to_fp16(src):
+    src = _u16(src)
+    d_src, d_dst = DevBuf.from_host(src), DevBuf(src.shape, np.uint16)
+    check(lib().llm_bf16_to_fp16(d_src.ptr, d_dst.ptr, src.size, None))
+    return d_dst.download()
+
+
+def embed_gather(table, ids):
+    table = _u16(table)
+    ids = np.ascontiguousarray(ids, dtype=np.int32)
+    vocab, d = table.shape
+    d_t, d_i, d_o = DevBuf.from_host(table), DevBuf.from_host(ids), DevBuf((ids.size, d), np.uint16)
+    check(lib().llm_embed_gather(d_t.ptr, d_i.ptr, None, d_o.ptr, ids.size, d, vocab, None))
+    return d_o.download()
+
+
+def rmsnorm(x, gain, eps=1e-5, inplace=False):
+    x, gain = _u16(x), _u16(gain)
+    T, d = x.shape
+    d_x, d_g = DevBuf.from_host(x), DevBuf.from_host(gain)
+    d_y = d_x if inplace else DevBuf(x.shape, np.uint16)
+    check(lib().llm_rmsnorm(d_x.ptr, d_g.ptr, d_y.ptr, T, d, eps, None))
+    return d_y.download()
+
+
+def add_residual(x, res):
+    x, res = _u16(x), _u16(res)
+    d_x, d_r = DevBuf.from_host(x), DevBuf.from_host(res)
+    check(lib().llm_add_residual(d_x.ptr, d_r.ptr, x.size, None))
+    return d_x.download()
+
+
+def rope_table(max_pos, head_dim, theta=500000.0):
+    tab = np.empty((max_pos, head_dim // 2, 2), np.float32)
+    check(lib().llm_rope_table_host(tab.ctypes.data, max_pos, head_dim, theta))
+    return tab
+
+
+def rope(buf, n_heads, head_dim, pos0=0, theta=500000.0, max_pos=None):
+    buf = _u16(buf)
+    T = buf.shape[0]
+    stride = buf.size // T
+    max_pos = max_pos or (pos0 + T + 63) // 64 * 64
+    d_b = DevBuf.from_host(buf)
+    d_t = DevBuf.from_host(rope_table(max_pos, head_dim, theta))
+    check(lib().llm_rope(d_b.ptr, T, n_heads, head_dim, stride, pos0, None, d_t.ptr, max_pos, None))
+    return d_b.download()
+
+
+def linear(x, w, residual=None):
+    x, w = _u16(x), _u16(w)
+    T, K = x.shape
+    N = w.shape[0]
+    d_x, d_w, d_o = DevBuf.from_host(x), DevBuf.from_host(w), DevBuf((T, N), np.uint16)
+    d_r = DevBuf.from_host(_u16(residual)) if residual is not None else None
+    check(lib().llm_linear(d_x.ptr, K, d_w.ptr, d_r.ptr if d_r else None, N, d_o.ptr, N, T, N, K, None))
+    return d_o.download()
+
+
+def linear_swiglu(x, wgate, wup):
+    x, wgate, wup = _u16(x), _u16(wgate), _u16(wup)
+    T, K = x.shape
+    N = wgate.shape[0]
+    d_x, d_g, d_u = DevBuf.from_host(x), DevBuf.from_host(wgate), DevBuf.from_host(wup)
+    d_o = DevBuf((T, N), np.uint16)
+    check(lib().llm_linear_swiglu(d_x.ptr, K, d_g.ptr, d_u.ptr, d_o.ptr, N, T, N, K, None))
+    return d_o.download()
+
+
+def kv_layout(k, v, n_kv_heads, head_dim, max_pos):
+    """token-major k, v [P, Hkv*hd] -> cache layouts K [Hkv][max_pos][hd], V [Hkv][hd][max_pos]."""
+    k, v = _u16(k), _u16(v)
+    P = k.shape[0]
+    kc = np.zeros((n_kv_heads, max_pos, head_dim), np.uint16)
+    vc = np.zeros((n_kv_heads, head_dim, max_pos), np.uint16)
+    kc[:, :P, :] = k.reshape(P, n_kv_heads, head_dim).transpose(1, 0, 2)
+    vc[:, :, :P] = v.reshape(P, n_kv_heads, head_dim).transpose(1, 2, 0)
+    return kc, vc
+
+
+def rope_kv_append(qkv, n_heads, n_kv_heads, head_dim, pos0, max_pos, theta=500000.0, kc=None, vc=None):
+    """Returns (qkv after the in-place Q rotation, K cache, V cache)."""
+    qkv = _u16(qkv)
+    T = qkv.shape[0]
+    kc = np.zeros((n_kv_heads, max_pos, head_dim), np.uint16) if kc is None else _u16(kc)
+    vc = np.zeros((n_kv_heads, head_dim, max_pos), np.uint16) if vc is None else _u16(vc)
+    d_q, d_k, d_v = DevBuf.from_host(qkv), DevBuf.from_host(kc), DevBuf.from_host(vc)
+    d_t = DevBuf.from_host(rope_table(max_pos, head_dim, theta))
+    check(lib().llm_rope_kv_append(d_q.ptr, d_k.ptr, d_v.ptr, T, n_heads, n_kv_heads, head_dim, pos0, None,
+                                   d_t.ptr, max_pos, None))
+    return d_q.download(), d_k.download(), d_v.download()
+
+
+def attn_decode(q, kc, vc, ctx, n_heads, n_kv_heads, head_dim, repeats=1):
+    q, kc, vc = _u16(q), _u16(kc), _u16(vc)
+    max_pos = kc.shape[1]
+    d_q, d_k, d_v = DevBuf.from_host(q), DevBuf.from_host(kc), DevBuf.from_host(vc)
+    d_o = DevBuf((n_heads * head_dim,), np.uint16)
+    wsb = (lib().llm_attn_decode_workspace_bytes(n_heads, head_dim) + 3) // 4 * 4
+    d_ws = DevBuf((wsb // 4,), np.uint32)
+    d_ws.zero()
+    for _ in range(repeats):  # the workspace is reusable without clearing
+        check(lib().llm_attn_decode(d_q.ptr, d_k.ptr, d_v.ptr, d_o.ptr, ctx, None, n_heads, n_kv_heads, head_dim,
+                                    max_pos, d_ws.ptr, None))
+    return d_o.download()
+
+
+def attn_prefill(q, kc, vc, pos0, n_heads, n_kv_heads, head_dim):
+    q, kc, vc = _u16(q), _u16(kc), _u16(vc)
+    T = q.shape[0]
+    ldq = q.size // T
+    max_pos = kc.shape[1]
+    d_q, d_k, d_v = DevBuf.from_host(q), DevBuf.from_host(kc), DevBuf.from_host(vc)
+    d_o = DevBuf((T, n_heads * head_dim), np.uint16)
+    check(lib().llm_attn_prefill(d_q.ptr, ldq, d_k.ptr, d_v.ptr, d_o.ptr, n_heads * head_dim, T, pos0, n_heads,
+                                 n_kv_heads, head_dim, max_pos, None))
+    return d_o.download()
+
+
+def lmhead_argmax(x, w):
+    """Returns (token, logits uint16[vocab])."""
+    x, w = _u16(x).reshape(-1), _u16(w)
+    vocab, K = w.shape
+    d_x, d_w = DevBuf.from_host(x), DevBuf.from_host(w)
+    d_l, d_t = DevBuf((vocab,), np.uint16), DevBuf((1,), np.int32)
+    d_ws = DevBuf((lib().llm_lmhead_workspace_bytes(vocab),), np.uint8)
+    check(lib().llm_lmhead_argmax(d_x.ptr, d_w.ptr, d_l.ptr, d_t.ptr, None, None, vocab, K, d_ws.ptr, None))
+    return int(d_t.download()[0]), d_l.download()
+
+
+def argmax_f16(logits):
+    logits = _u16(logits).reshape(-1)
+    d_l, d_t = DevBuf.from_host(logits), DevBuf((1,), np.int32)
+    d_ws = DevBuf((lib().llm_lmhead_workspace_bytes(logits.size),), np.uint8)
+    check(lib().llm_argmax_f16(d_l.ptr, logits.size, d_t.ptr, d_ws.ptr, None))
+    return int(d_t.download()[0])
+
+
+class Timer:
+    """HIP-event timing of repeated launches on one stream."""
+
+    def __init__(self):
+        capi.require_gpu()
+        self.stream = C.c_void_p()
+        check(lib().llm_stream_create(C.byref(self.stream)))
+        self.e0, self.e1 = C.c_void_p(), C.c_void_p()
+        check(lib().llm_event_create(C.byref(self.e0)))
+        check(lib().llm_event_create(C.byref(self.e1)))
+
+    def time(self, fn, iters=20, warmup=3):
+        """fn(stream) issues the launches; returns mean milliseconds per call."""
+        for _ in range(warmup):
+            fn(self.stream)
+        check(lib().llm_stream_sync(self.stream))
+        check(lib().llm_event_record(self.e0, self.stream))
+        for _ in range(iters):
+            fn(self.stream)
+        check(lib().llm_event_record(self.e1, self.stream))
+        check(lib().llm_event_sync(self.e1))
+        ms = C.c_float(0)
+        check(lib().llm_event_elapsed_ms(self.e0, self.e1, C.byref(ms)))
+        return ms.value / iters

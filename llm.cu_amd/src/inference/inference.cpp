@@ -1,0 +1,422 @@
+// Forward / generation driver.  Keeps the reference's entry points
+// (init_cache, inference; src/inference/inference.cu:110-193) and adds what the
+// token loop needs on top: an fp16 KV cache, a prompt pass that processes many
+// rows at once, a one-row decode step captured as a hipGraph, greedy argmax on
+// the device.  All device work goes through llmcu_hip.h.
+//
+// Layer graph (inference.cu:157-186), with the reference's extra passes folded
+// into neighbours where the result is the same bits:
+//   save residual + norm      -> llm_rmsnorm into a second buffer (x stays the residual)
+//   Q, K, V (3 launches)      -> one projection over the adjacent q|k|v weights
+//   RoPE(Q), RoPE(K)          -> llm_rope_kv_append (also writes the KV cache)
+//   scores, softmax, P.V      -> llm_attn_prefill / llm_attn_decode over the cache
+//   copy + O projection, add  -> llm_linear with the residual in its epilogue
+//   gate/up+SiLU, down, add   -> llm_linear_swiglu, llm_linear with residual
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <vector>
+
+#include "common/fail.h"
+#include "llama3/llama3.h"
+#include "llama3_host.h"
+#include "llmcu_hip.h"
+
+namespace {
+
+struct Engine {
+    ModelConfig cfg;
+    llm_stream_t stream = nullptr;
+    int qkv_dim = 0;
+    // activations, sized for max_pos rows
+    llm_half *x = nullptr, *xn = nullptr, *qkv = nullptr, *attn = nullptr, *ffn = nullptr;
+    llm_half *logits = nullptr;
+    // KV cache: K [L][Hkv][max_pos][hd], V [L][Hkv][hd][max_pos]
+    llm_half *kc = nullptr, *vc = nullptr;
+    size_t kv_layer_elems = 0;
+    float *rope_table = nullptr;
+    int32_t *d_tokens = nullptr; // [max_pos + 1]
+    int32_t *d_pos = nullptr;    // tokens cached so far; d_tokens[*d_pos] is the next input
+    int32_t *d_token = nullptr;  // last argmax
+    void *ws_attn = nullptr, *ws_lm = nullptr;
+    llm_half *trace_dev = nullptr;
+    size_t trace_rows = 0;
+    llm_half *trace_host = nullptr;
+    std::vector<int> tokens; // ids whose K/V are cached
+    int pos = 0;
+    bool use_graph = true;
+    llm_graph_t graph = nullptr;
+    llm_event_t ev[4] = {nullptr, nullptr, nullptr, nullptr};
+};
+
+Engine *eng(const CudaCache *c) {
+    if (!c || !c->engine) llama3_fail("CudaCache was not created by init_cache");
+    return (Engine *)c->engine;
+}
+
+template <typename T> T *dmalloc(size_t n, const char *what) {
+    void *p = nullptr;
+    llama3_check(llm_malloc(&p, n * sizeof(T)), what);
+    return (T *)p;
+}
+
+struct LayerW {
+    const llm_half *in_ln, *post_ln, *wq, *wk, *wv, *wo, *wg, *wu, *wd;
+};
+
+LayerW layer_w(const Llama3 *m, int l) {
+    const Llama3Layer *L = m->layers[l];
+    return {L->input_layernorm->d_fp16_tensor,  L->post_attention_layernorm->d_fp16_tensor,
+            L->self_attn_q_proj->d_fp16_tensor, L->self_attn_k_proj->d_fp16_tensor,
+            L->self_attn_v_proj->d_fp16_tensor, L->self_attn_o_proj->d_fp16_tensor,
+            L->mlp_gate_proj->d_fp16_tensor,    L->mlp_up_proj->d_fp16_tensor,
+            L->mlp_down_proj->d_fp16_tensor};
+}
+
+void check_shapes(const Llama3 *m, const ModelConfig &c) {
+    auto want = [](const Tensor *t, int r, int cc, const char *name) {
+        if (!t || !t->shape || !t->d_fp16_tensor) llama3_fail("%s is not on the device (call to_cuda first)", name);
+        int rows = t->shape[0], cols = *t->ndim > 1 ? t->shape[1] : 0;
+        if (rows != r || cols != cc) llama3_fail("%s is [%d,%d], the configuration needs [%d,%d]", name, rows, cols, r, cc);
+    };
+    const int d = c.d_model, qd = c.n_heads * c.head_dim, kvd = c.n_kv_heads * c.head_dim;
+    if (m->n_layers != c.n_layers) llama3_fail("model has %d layers, configuration %d", m->n_layers, c.n_layers);
+    want(m->embed_tokens, c.vocab, d, "embed_tokens");
+    want(m->lm_head, c.vocab, d, "lm_head");
+    want(m->norm, d, 0, "norm");
+    for (int l = 0; l < c.n_layers; ++l) {
+        const Llama3Layer *L = m->layers[l];
+        want(L->input_layernorm, d, 0, "input_layernorm");
+        want(L->post_attention_layernorm, d, 0, "post_attention_layernorm");
+        want(L->self_attn_q_proj, qd, d, "q_proj");
+        want(L->self_attn_k_proj, kvd, d, "k_proj");
+        want(L->self_attn_v_proj, kvd, d, "v_proj");
+        want(L->self_attn_o_proj, d, qd, "o_proj");
+        want(L->mlp_gate_proj, c.ffn_dim, d, "gate_proj");
+        want(L->mlp_up_proj, c.ffn_dim, d, "up_proj");
+        want(L->mlp_down_proj, d, c.ffn_dim, "down_proj");
+    }
+}
+
+// Issues one pass over T rows on the engine's stream.  With dev_pos the row
+// position comes from *d_pos (T must be 1): that form is what gets captured.
+void issue_pass(Engine *e, const Llama3 *m, int T, int pos0, bool dev_pos, bool trace) {
+    const ModelConfig &c = e->cfg;
+    const int d = c.d_model, hd = c.head_dim, Hq = c.n_heads, Hkv = c.n_kv_heads, F = c.ffn_dim;
+    const int qd = Hq * hd, kvd = Hkv * hd, QKV = e->qkv_dim;
+    llm_stream_t s = e->stream;
+    const int32_t *pd = dev_pos ? e->d_pos : nullptr;
+    const int p0 = dev_pos ? 0 : pos0;
+
+    llama3_check(llm_embed_gather(m->embed_tokens->d_fp16_tensor, e->d_tokens + p0, pd, e->x, T, d, c.vocab, s),
+                 "llm_embed_gather");
+    for (int l = 0; l < c.n_layers; ++l) {
+        const LayerW w = layer_w(m, l);
+        llm_half *kc = e->kc + (size_t)l * e->kv_layer_elems, *vc = e->vc + (size_t)l * e->kv_layer_elems;
+        llama3_check(llm_rmsnorm(e->x, w.in_ln, e->xn, T, d, c.rms_eps, s), "llm_rmsnorm");
+        if (w.wk == w.wq + (size_t)qd * d && w.wv == w.wk + (size_t)kvd * d) {
+            llama3_check(llm_linear(e->xn, d, w.wq, nullptr, 0, e->qkv, QKV, T, QKV, d, s), "llm_linear(qkv)");
+        } else {
+            llama3_check(llm_linear(e->xn, d, w.wq, nullptr, 0, e->qkv, QKV, T, qd, d, s), "llm_linear(q)");
+            llama3_check(llm_linear(e->xn, d, w.wk, nullptr, 0, e->qkv + qd, QKV, T, kvd, d, s), "llm_linear(k)");
+            llama3_check(llm_linear(e->xn, d, w.wv, nullptr, 0, e->qkv + qd + kvd, QKV, T, kvd, d, s), "llm_linear(v)");
+        }
+        llama3_check(llm_rope_kv_append(e->qkv, kc, vc, T, Hq, Hkv, hd, p0, pd, e->rope_table, c.max_pos, s),
+                     "llm_rope_kv_append");
+        if (T == 1) {
+            llama3_check(llm_attn_decode(e->qkv, kc, vc, e->attn, p0 + 1, pd, Hq, Hkv, hd, c.max_pos, e->ws_attn, s),
+                         "llm_attn_decode");
+        } else {
+            llama3_check(llm_attn_prefill(e->qkv, QKV, kc, vc, e->attn, qd, T, p0, Hq, Hkv, hd, c.max_pos, s),
+                         "llm_attn_prefill");
+        }
+        llama3_check(llm_linear(e->attn, qd, w.wo, e->x, d, e->x, d, T, d, qd, s), "llm_linear(o)");
+        llama3_check(llm_rmsnorm(e->x, w.post_ln, e->xn, T, d, c.rms_eps, s), "llm_rmsnorm");
+        llama3_check(llm_linear_swiglu(e->xn, d, w.wg, w.wu, e->ffn, F, T, F, d, s), "llm_linear_swiglu");
+        llama3_check(llm_linear(e->ffn, F, w.wd, e->x, d, e->x, d, T, d, F, s), "llm_linear(down)");
+        if (trace)
+            llama3_check(llm_memcpy_d2d(e->trace_dev + (size_t)l * T * d, e->x, sizeof(llm_half) * (size_t)T * d, s),
+                         "trace copy");
+    }
+    // final norm on the last row only (the reference norms all rows and reads the last)
+    llama3_check(llm_rmsnorm(e->x + (size_t)(T - 1) * d, m->norm->d_fp16_tensor, e->xn, 1, d, c.rms_eps, s),
+                 "llm_rmsnorm(final)");
+    llama3_check(llm_lmhead_argmax(e->xn, m->lm_head->d_fp16_tensor, e->logits, e->d_token, e->d_tokens, e->d_pos,
+                                   c.vocab, d, e->ws_lm, s),
+                 "llm_lmhead_argmax");
+}
+
+void drop_graph(Engine *e) {
+    if (e->graph) {
+        llm_graph_destroy(e->graph);
+        e->graph = nullptr;
+    }
+}
+
+// Appends n host tokens at e->pos with one multi-row pass.  Leaves
+// d_pos = pos + n and d_tokens[pos + n] = the greedy next token.
+int run_pass(Engine *e, const Llama3 *m, const int *tokens, int n) {
+    const ModelConfig &c = e->cfg;
+    if (n < 1) llama3_fail("a pass needs at least one token");
+    if (e->pos + n > c.max_pos) llama3_fail("sequence of %d tokens exceeds max_pos %d", e->pos + n, c.max_pos);
+    for (int i = 0; i < n; ++i)
+        if (tokens[i] < 0 || tokens[i] >= c.vocab) llama3_fail("token id %d outside the vocabulary", tokens[i]);
+    llm_stream_t s = e->stream;
+    llama3_check(llm_memcpy_h2d(e->d_tokens + e->pos, tokens, sizeof(int) * (size_t)n, s), "H2D tokens");
+    const int32_t last = e->pos + n - 1;
+    llama3_check(llm_memcpy_h2d(e->d_pos, &last, sizeof(int32_t), s), "H2D position");
+    llama3_check(llm_stream_sync(s), "stream sync"); // `last` is a stack variable
+    const bool trace = e->trace_host != nullptr;
+    if (trace) {
+        size_t need = (size_t)c.n_layers * n * c.d_model;
+        if (need > e->trace_rows) {
+            if (e->trace_dev) llm_free(e->trace_dev);
+            e->trace_dev = dmalloc<llm_half>(need, "llm_malloc(trace)");
+            e->trace_rows = need;
+        }
+    }
+    issue_pass(e, m, n, e->pos, false, trace);
+    int32_t tok = -1;
+    llama3_check(llm_memcpy_d2h(&tok, e->d_token, sizeof(int32_t), s), "D2H token");
+    if (trace)
+        llama3_check(llm_memcpy_d2h(e->trace_host, e->trace_dev, sizeof(llm_half) * (size_t)c.n_layers * n * c.d_model, s),
+                     "D2H trace");
+    llama3_check(llm_stream_sync(s), "stream sync");
+    e->trace_host = nullptr;
+    e->tokens.insert(e->tokens.end(), tokens, tokens + n);
+    e->pos += n;
+    return (int)tok;
+}
+
+// One decode step from device state (d_tokens[*d_pos] in, next token out).
+void launch_decode_step(Engine *e, const Llama3 *m) {
+    if (e->use_graph) {
+        if (!e->graph) {
+            llama3_check(llm_graph_capture_begin(e->stream), "graph capture begin");
+            issue_pass(e, m, 1, 0, true, false);
+            llama3_check(llm_graph_capture_end(e->stream, &e->graph), "graph capture end");
+        }
+        llama3_check(llm_graph_launch(e->graph, e->stream), "graph launch");
+    } else {
+        issue_pass(e, m, 1, 0, true, false);
+    }
+}
+
+} // namespace
+
+// ---------------------------------------------------------------------------
+extern "C" CudaCache *init_cache_cfg(Llama3 *m, const ModelConfig *cfg) {
+    const ModelConfig &c = *cfg;
+    if (c.max_pos <= 0 || c.max_pos % 64) llama3_fail("max_pos %d must be a positive multiple of 64", c.max_pos);
+    if (c.n_kv_heads <= 0 || c.n_heads % c.n_kv_heads) llama3_fail("heads %d/%d", c.n_heads, c.n_kv_heads);
+    check_shapes(m, c);
+    Engine *e = new Engine;
+    e->cfg = c;
+    const int d = c.d_model, qd = c.n_heads * c.head_dim, kvd = c.n_kv_heads * c.head_dim;
+    e->qkv_dim = qd + 2 * kvd;
+    const size_t R = (size_t)c.max_pos;
+    llama3_check(llm_stream_create(&e->stream), "llm_stream_create");
+    e->x = dmalloc<llm_half>(R * d, "llm_malloc(x)");
+    e->xn = dmalloc<llm_half>(R * d, "llm_malloc(xn)");
+    e->qkv = dmalloc<llm_half>(R * e->qkv_dim, "llm_malloc(qkv)");
+    e->attn = dmalloc<llm_half>(R * qd, "llm_malloc(attn)");
+    e->ffn = dmalloc<llm_half>(R * c.ffn_dim, "llm_malloc(ffn)");
+    e->logits = dmalloc<llm_half>((size_t)c.vocab, "llm_malloc(logits)");
+    e->kv_layer_elems = (size_t)c.n_kv_heads * R * c.head_dim;
+    e->kc = dmalloc<llm_half>(e->kv_layer_elems * c.n_layers, "llm_malloc(K cache)");
+    e->vc = dmalloc<llm_half>(e->kv_layer_elems * c.n_layers, "llm_malloc(V cache)");
+    llama3_check(llm_fill_zero(e->kc, sizeof(llm_half) * e->kv_layer_elems * c.n_layers, e->stream), "zero K cache");
+    llama3_check(llm_fill_zero(e->vc, sizeof(llm_half) * e->kv_layer_elems * c.n_layers, e->stream), "zero V cache");
+    {
+        size_t n = R * (c.head_dim / 2) * 2;
+        std::vector<float> tab(n);
+        llama3_check(llm_rope_table_host(tab.data(), c.max_pos, c.head_dim, c.rope_theta), "llm_rope_table_host");
+        e->rope_table = dmalloc<float>(n, "llm_malloc(rope table)");
+        llama3_check(llm_memcpy_h2d(e->rope_table, tab.data(), sizeof(float) * n, nullptr), "H2D rope table");
+    }
+    e->d_tokens = dmalloc<int32_t>(R + 1, "llm_malloc(tokens)");
+    e->d_pos = dmalloc<int32_t>(1, "llm_malloc(pos)");
+    e->d_token = dmalloc<int32_t>(1, "llm_malloc(token)");
+    llama3_check(llm_fill_zero(e->d_tokens, sizeof(int32_t) * (R + 1), e->stream), "zero tokens");
+    llama3_check(llm_fill_zero(e->d_pos, sizeof(int32_t), e->stream), "zero pos");
+    size_t wa = llm_attn_decode_workspace_bytes(c.n_heads, c.head_dim);
+    wa = (wa + 3) / 4 * 4;
+    llama3_check(llm_malloc(&e->ws_attn, wa), "llm_malloc(attention workspace)");
+    llama3_check(llm_fill_zero(e->ws_attn, wa, e->stream), "zero attention workspace");
+    llama3_check(llm_malloc(&e->ws_lm, llm_lmhead_workspace_bytes(c.vocab)), "llm_malloc(lm head workspace)");
+    for (auto &ev : e->ev) llama3_check(llm_event_create(&ev), "llm_event_create");
+    llama3_check(llm_stream_sync(e->stream), "stream sync");
+
+    CudaCache *C = (CudaCache *)calloc(1, sizeof(CudaCache));
+    if (!C) llama3_fail("Memory allocation failed for CudaCache");
+    C->d_feedforward_cache_upgate = e->ffn;
+    C->d_token_probdist = e->logits;
+    C->h_token_probdist = (llm_half *)malloc(sizeof(llm_half) * (size_t)c.vocab);
+    C->f_token_probdist = (float *)malloc(sizeof(float) * (size_t)c.vocab);
+    C->engine = e;
+    return C;
+}
+
+// inference.cu:110-145.  Shapes come from the loaded tensors; head_dim 128 and
+// the 2048-token limit are the reference's constants (inference.cu:122,700).
+extern "C" CudaCache *init_cache(Llama3 *m) {
+    ModelConfig c = llama3_config_8b();
+    if (!m || !m->embed_tokens || !m->embed_tokens->shape) llama3_fail("init_cache: the model holds no tensors");
+    c.n_layers = m->n_layers;
+    c.vocab = m->embed_tokens->shape[0];
+    c.d_model = m->embed_tokens->shape[1];
+    c.ffn_dim = m->layers[0]->mlp_gate_proj->shape[0];
+    c.head_dim = 128;
+    c.n_heads = m->layers[0]->self_attn_q_proj->shape[0] / c.head_dim;
+    c.n_kv_heads = m->layers[0]->self_attn_k_proj->shape[0] / c.head_dim;
+    c.max_pos = 2048;
+    return init_cache_cfg(m, &c);
+}
+
+extern "C" void free_cache(CudaCache *C) {
+    if (!C) return;
+    Engine *e = (Engine *)C->engine;
+    if (e) {
+        llm_stream_sync(e->stream);
+        drop_graph(e);
+        void *bufs[] = {e->x, e->xn, e->qkv, e->attn, e->ffn, e->logits, e->kc, e->vc, e->rope_table,
+                        e->d_tokens, e->d_pos, e->d_token, e->ws_attn, e->ws_lm, e->trace_dev};
+        for (void *b : bufs) llm_free(b);
+        for (auto ev : e->ev) llm_event_destroy(ev);
+        llm_stream_destroy(e->stream);
+        delete e;
+    }
+    free(C->h_token_probdist);
+    free(C->f_token_probdist);
+    free(C);
+}
+
+// tokenizer.cu:157-198: the activation tensor X ([2048, embed] fp16, zeroed)
+// and the device token array.  The engine keeps its own activations; X and
+// d_tokens exist so that callers written for the reference keep working.
+extern "C" int *tokens_to_cuda(int *tokens, int embed_size, Tensor *X) {
+    (void)tokens;
+    memset(X, 0, sizeof(Tensor));
+    int shape[2] = {2048, embed_size};
+    tensor_set_host_shape(X, 2, shape);
+    void *p = nullptr;
+    llama3_check(llm_malloc(&p, sizeof(llm_half) * (size_t)*X->mem_len), "llm_malloc(X)");
+    X->d_fp16_tensor = (llm_half *)p;
+    llama3_check(llm_fill_zero(p, sizeof(llm_half) * (size_t)*X->mem_len, nullptr), "zero X");
+    void *dt = nullptr;
+    llama3_check(llm_malloc(&dt, sizeof(int) * 2048), "llm_malloc(d_tokens)");
+    llama3_check(llm_device_sync(), "device sync");
+    return (int *)dt;
+}
+
+extern "C" void llama3_cache_reset(CudaCache *C) {
+    Engine *e = eng(C);
+    e->pos = 0;
+    e->tokens.clear();
+}
+
+extern "C" int llama3_cache_pos(const CudaCache *C) { return eng(C)->pos; }
+
+extern "C" int llama3_prefill(Llama3 *m, CudaCache *C, const int *tokens, int n) {
+    return run_pass(eng(C), m, tokens, n);
+}
+
+extern "C" int llama3_decode(Llama3 *m, CudaCache *C, int token) {
+    Engine *e = eng(C);
+    if (e->trace_host) return run_pass(e, m, &token, 1);
+    const ModelConfig &c = e->cfg;
+    if (e->pos + 1 > c.max_pos) llama3_fail("sequence of %d tokens exceeds max_pos %d", e->pos + 1, c.max_pos);
+    if (token < 0 || token >= c.vocab) llama3_fail("token id %d outside the vocabulary", token);
+    llm_stream_t s = e->stream;
+    const int32_t p = e->pos, t = token;
+    llama3_check(llm_memcpy_h2d(e->d_tokens + e->pos, &t, sizeof(int32_t), s), "H2D token");
+    llama3_check(llm_memcpy_h2d(e->d_pos, &p, sizeof(int32_t), s), "H2D position");
+    llama3_check(llm_stream_sync(s), "stream sync");
+    launch_decode_step(e, m);
+    int32_t tok = -1;
+    llama3_check(llm_memcpy_d2h(&tok, e->d_token, sizeof(int32_t), s), "D2H token");
+    llama3_check(llm_stream_sync(s), "stream sync");
+    e->tokens.push_back(token);
+    e->pos += 1;
+    return (int)tok;
+}
+
+extern "C" int llama3_generate(Llama3 *m, CudaCache *C, const int *prompt, int n_prompt, int n_decode,
+                               int *out_tokens, GenStats *stats) {
+    Engine *e = eng(C);
+    const ModelConfig &c = e->cfg;
+    if (n_decode < 1) llama3_fail("llama3_generate: n_decode must be at least 1");
+    if (e->pos + n_prompt + n_decode - 1 > c.max_pos)
+        llama3_fail("prompt %d + %d decode steps exceed max_pos %d", e->pos + n_prompt, n_decode - 1, c.max_pos);
+    llm_stream_t s = e->stream;
+    const int start = e->pos;
+    llama3_check(llm_event_record(e->ev[0], s), "event record");
+    int first = run_pass(e, m, prompt, n_prompt); // syncs
+    llama3_check(llm_event_record(e->ev[1], s), "event record");
+    // capture outside the timed decode region
+    if (e->use_graph && !e->graph && n_decode > 1) {
+        llama3_check(llm_graph_capture_begin(s), "graph capture begin");
+        issue_pass(e, m, 1, 0, true, false);
+        llama3_check(llm_graph_capture_end(s, &e->graph), "graph capture end");
+    }
+    llama3_check(llm_event_record(e->ev[2], s), "event record");
+    for (int i = 1; i < n_decode; ++i) launch_decode_step(e, m);
+    llama3_check(llm_event_record(e->ev[3], s), "event record");
+    llama3_check(llm_stream_sync(s), "stream sync");
+    out_tokens[0] = first;
+    if (n_decode > 1) {
+        llama3_check(llm_memcpy_d2h(out_tokens + 1, e->d_tokens + start + n_prompt + 1,
+                                    sizeof(int32_t) * (size_t)(n_decode - 1), s),
+                     "D2H tokens");
+        llama3_check(llm_stream_sync(s), "stream sync");
+    }
+    // host mirror: the decode steps consumed out_tokens[0..n_decode-2]
+    for (int i = 0; i + 1 < n_decode; ++i) e->tokens.push_back(out_tokens[i]);
+    e->pos += n_decode - 1;
+    if (stats) {
+        float a = 0.f, b = 0.f;
+        llm_event_elapsed_ms(e->ev[0], e->ev[1], &a);
+        llm_event_elapsed_ms(e->ev[2], e->ev[3], &b);
+        stats->prefill_ms = a;
+        stats->decode_ms = b;
+        stats->n_prompt = n_prompt;
+        stats->n_decode_steps = n_decode - 1;
+    }
+    return 0;
+}
+
+extern "C" void llama3_set_hidden_trace(CudaCache *C, llm_half *hidden) { eng(C)->trace_host = hidden; }
+
+extern "C" void llama3_read_logits(CudaCache *C, llm_half *logits) {
+    Engine *e = eng(C);
+    llama3_check(llm_memcpy_d2h(logits, e->logits, sizeof(llm_half) * (size_t)e->cfg.vocab, e->stream), "D2H logits");
+    llama3_check(llm_stream_sync(e->stream), "stream sync");
+}
+
+extern "C" void llama3_set_use_graph(CudaCache *C, int on) {
+    Engine *e = eng(C);
+    e->use_graph = on != 0;
+    if (!e->use_graph) drop_graph(e);
+}
+
+// inference.cu:149-193.  h_tokens[0] = n + 1, ids in h_tokens[1..n].  The
+// reference recomputes all n rows on every call; here rows whose K/V are
+// already cached (same leading ids as the previous call) are not recomputed,
+// which yields the same next token because the recompute is causal.
+extern "C" int inference(Llama3 *m, Tensor *X, int *d_tokens, int *h_tokens, CudaCache *C) {
+    (void)X;
+    Engine *e = eng(C);
+    const int n = h_tokens[0] - 1;
+    const int *ids = h_tokens + 1;
+    if (n < 1) llama3_fail("inference: empty token list");
+    if (d_tokens) // the reference's H2D of the whole token array (inference.cu:150)
+        llama3_check(llm_memcpy_h2d(d_tokens, h_tokens, sizeof(int) * (size_t)(n + 1 < 2048 ? n + 1 : 2048), nullptr),
+                     "H2D tokens");
+    bool extend = n > e->pos;
+    for (int i = 0; extend && i < e->pos; ++i) extend = ids[i] == e->tokens[i];
+    if (!extend) llama3_cache_reset(C);
+    const int fresh = n - e->pos;
+    int tok = fresh == 1 ? llama3_decode(m, C, ids[n - 1]) : llama3_prefill(m, C, ids + e->pos, fresh);
+    llama3_read_logits(C, C->h_token_probdist);
+    return tok;
+}

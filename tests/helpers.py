@@ -1,0 +1,154 @@
+"""Shared pieces of the parity tests: numpy float64 closed forms, the mixed
+abs/rel error the north star states (2e-2), and the whole-model comparison of
+the HIP engine with the CPU oracle on identical seeded weights."""
+import numpy as np
+
+from oracle import pyoracle as orc
+
+TOL = 2e-2  # max-abs/rel tolerance for fp16 hidden states and logits
+
+
+def f16(bits):
+    return np.ascontiguousarray(bits).view(np.float16).astype(np.float64)
+
+
+def bits(a):
+    return np.ascontiguousarray(np.asarray(a, dtype=np.float16)).view(np.uint16)
+
+
+def mixed_err(a_bits, b_bits):
+    """max_i |a-b| / max(1, |b|): absolute below magnitude 1, relative above."""
+    a, b = f16(a_bits), f16(b_bits)
+    return float(np.max(np.abs(a - b) / np.maximum(1.0, np.abs(b)))) if a.size else 0.0
+
+
+def ulp_diff(a_bits, b_bits):
+    """distance in fp16 ulps (monotone integer mapping of the bit patterns)."""
+    def key(x):
+        x = np.ascontiguousarray(x).astype(np.int32)
+        return np.where(x & 0x8000, -(x & 0x7fff), x & 0x7fff)
+    return np.abs(key(a_bits) - key(b_bits))
+
+
+def bf16_to_f32(b):
+    return (np.ascontiguousarray(b).astype(np.uint32) << 16).view(np.float32)
+
+
+def f32_to_bf16(x):
+    u = np.ascontiguousarray(x, dtype=np.float32).view(np.uint32)
+    return ((u + 0x7fff + ((u >> 16) & 1)) >> 16).astype(np.uint16)
+
+
+def cfg_dict(cfg):
+    return {k: getattr(cfg, k) for k, _ in cfg._fields_}
+
+
+def oracle_weights(model):
+    """fp16 weights for the oracle from a host-side (not yet uploaded) Model:
+    the oracle's own BF16->FP16 over the same bf16 bits the GPU will convert."""
+    h = model.host_bf16()
+    conv = lambda a: orc.bf16_to_fp16(np.ascontiguousarray(a).reshape(-1)).reshape(a.shape)
+    return {
+        "embed": conv(h["embed"]), "lm_head": conv(h["lm_head"]), "norm": conv(h["norm"]),
+        "input_ln": [conv(a) for a in h["input_layernorm"]],
+        "post_ln": [conv(a) for a in h["post_attention_layernorm"]],
+        "wq": [conv(a) for a in h["self_attn_q_proj"]],
+        "wk": [conv(a) for a in h["self_attn_k_proj"]],
+        "wv": [conv(a) for a in h["self_attn_v_proj"]],
+        "wo": [conv(a) for a in h["self_attn_o_proj"]],
+        "wgate": [conv(a) for a in h["mlp_gate_proj"]],
+        "wup": [conv(a) for a in h["mlp_up_proj"]],
+        "wdown": [conv(a) for a in h["mlp_down_proj"]],
+    }
+
+
+def run_model_parity(pkg, cfg, seed, n_prompt, n_decode, use_graph=True, oracle_decode=None):
+    """Runs prompt + greedy decode on the HIP engine and on the ORC_REF16
+    oracle from the same seeded bf16 weights and prompt.  Returns errors and
+    both token sequences.  oracle_decode limits how many decode steps the
+    oracle follows (default: all)."""
+    eng_mod = pkg.engine
+    model = eng_mod.Model.seeded(cfg, seed)
+    w = oracle_weights(model)
+    model.to_device()
+    prompt = eng_mod.seeded_tokens(seed, n_prompt, cfg.vocab)
+    out = {}
+    # weight conversion must be bit-exact
+    dev_embed = model.device_fp16(model.handle.contents.embed_tokens)
+    out["convert_exact"] = bool(np.array_equal(dev_embed, w["embed"]))
+
+    engine = eng_mod.Engine(model, cfg, use_graph=use_graph)
+    o = orc.Model(cfg_dict(cfg), w, orc.ORC_REF16)
+
+    tok_g, hid_g = engine.prefill(prompt, want_hidden=True)
+    logits_g = engine.logits()
+    tok_o, hid_o, logits_o = o.forward(prompt, want_hidden=True)
+    out["hidden_max_err"] = max(mixed_err(hid_g[l], hid_o[l]) for l in range(cfg.n_layers))
+    out["hidden_err_per_layer"] = [mixed_err(hid_g[l], hid_o[l]) for l in range(cfg.n_layers)]
+    out["logits_max_err"] = mixed_err(logits_g, logits_o)
+    out["argmax_matches_own_logits"] = bool(tok_g == orc.argmax_f16(logits_g))
+    out["first_token"] = (int(tok_g), int(tok_o))
+
+    # greedy decode: device-resident loop vs oracle
+    engine.reset()
+    toks_g, stats = engine.generate(prompt, n_decode)
+    n_o = n_decode if oracle_decode is None else min(n_decode, oracle_decode)
+    toks_o = [int(tok_o)]
+    gaps = []
+    for _ in range(n_o - 1):
+        t, _, lg = o.forward([toks_o[-1]])
+        v = np.sort(f16(lg))
+        gaps.append(float(v[-1] - v[-2]))
+        toks_o.append(int(t))
+    out["tokens_gpu"] = [int(t) for t in toks_g[:n_o]]
+    out["tokens_oracle"] = toks_o
+    out["top2_gaps"] = gaps
+    out["stats"] = {"prefill_ms": stats.prefill_ms, "decode_ms": stats.decode_ms,
+                    "n_decode_steps": stats.n_decode_steps}
+    out["tokens_all_gpu"] = [int(t) for t in toks_g]
+    o.close()
+    engine.close()
+    model.close()
+    return out
+
+
+# ---- float64 closed forms ------------------------------------------------------
+def rmsnorm_f64(x, g, eps=1e-5):
+    x, g = f16(x), f16(g)
+    rms = np.sqrt(eps + np.mean(x * x, axis=-1, keepdims=True))
+    return x * g / rms
+
+
+def rope_f64(x, n_heads, head_dim, pos0=0, theta=500000.0):
+    x = f16(x).reshape(x.shape[0], n_heads, head_dim // 2, 2)
+    T = x.shape[0]
+    i = np.arange(head_dim // 2, dtype=np.float64)
+    freq = theta ** (-2.0 * i / head_dim)
+    ang = (pos0 + np.arange(T, dtype=np.float64))[:, None] * freq[None, :]
+    c, s = np.cos(ang)[:, None, :], np.sin(ang)[:, None, :]
+    e, o = x[..., 0], x[..., 1]
+    out = np.stack([c * e - s * o, s * e + c * o], axis=-1)
+    return out.reshape(T, n_heads * head_dim)
+
+
+def attention_f64(q, k, v, pos0, n_heads, n_kv_heads, head_dim):
+    q, k, v = f16(q), f16(k), f16(v)
+    Tq = q.shape[0]
+    g = n_heads // n_kv_heads
+    out = np.zeros_like(q)
+    for h in range(n_heads):
+        kv = h // g
+        qh = q[:, h * head_dim:(h + 1) * head_dim]
+        kh = k[:, kv * head_dim:(kv + 1) * head_dim]
+        vh = v[:, kv * head_dim:(kv + 1) * head_dim]
+        for t in range(Tq):
+            n = pos0 + t + 1
+            s = kh[:n] @ qh[t] / np.sqrt(head_dim)
+            p = np.exp(s - s.max())
+            p /= p.sum()
+            out[t, h * head_dim:(h + 1) * head_dim] = p @ vh[:n]
+    return out
+
+
+def silu(x):
+    return x / (1.0 + np.exp(-x))
