@@ -1,0 +1,205 @@
+#!/usr/bin/env python3
+"""Headline benchmark: LLaMA3-8B batch-1 greedy decode on one MI355X.
+
+A "step" is one decode token through all 32 layers + LM head + argmax with
+the KV cache and every weight resident in HBM.  The workload is the full
+LLaMA3-8B decoder of BASELINE.json (seeded random-init bf16 weights converted
+to fp16 at load, prompt of 128 seeded ids, then K greedy decode steps).  The
+same run also measures the 8192-token prompt pass (MFMA GEMM + causal GQA
+attention), the dominant kernel (fused gate/up SwiGLU GEMV) against the HBM
+roofline with HIP events, and the fp32 CPU port of the reference forward pass
+on the host cores as a reported baseline.
+
+    python bench.py [--gpus 1] [--steps 256] [--warmup 8]
+
+Prints ONE JSON line.
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK = 8.0e12          # B/s, MI355X HBM3E
+MFMA_F16_PEAK = 2.5e15     # flop/s, MI355X dense fp16
+
+
+def decode_bytes(ctx):
+    """Algorithmic HBM bytes of one decode token at context ctx (keys attended):
+    every layer's weights + LM head + final norm in fp16, K and V rows of ctx
+    positions, one new K/V row, one embedding row."""
+    params = 32 * 218112000 + 525336576 + 4096
+    return 2 * params + 131072 * ctx + 131072 + 8192
+
+
+def prefill_flops(T):
+    return 2.0 * T * 6979321856 + 262144.0 * T * (T + 1) + 2.0 * 4096 * 128256
+
+
+def log(*a):
+    print("[bench]", *a, file=sys.stderr, flush=True)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=256)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--prompt", type=int, default=128)
+    ap.add_argument("--seed", type=int, default=1234)
+    ap.add_argument("--no-prefill-8k", action="store_true")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-steps", type=int, default=8)
+    ap.add_argument("--no-graph", action="store_true")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        sys.exit("bench.py: this build measures one MI355X; --gpus %d is not supported "
+                 "(no collective path exists, every figure is the one GPU's)" % a.gpus)
+
+    import __graft_entry__ as ge
+    pkg = ge.load_package()
+    pkg.init(0)
+    lib = pkg.lib()
+    eng_mod = pkg.engine
+
+    cfg = eng_mod.config("8b", max_pos=8704)
+    t0 = time.time()
+    model = eng_mod.Model.seeded(cfg, a.seed)
+    log("seeded bf16 weights on the host in %.1f s" % (time.time() - t0))
+
+    orc = None
+    orc_w = None
+    if not a.no_cpu_baseline:
+        from oracle import pyoracle as orc
+        from tests import helpers as H
+        t0 = time.time()
+        orc_w = H.oracle_weights(model)  # fp16 copies for the CPU port, before to_cuda frees the bf16
+        log("fp16 host copy for the CPU baseline in %.1f s" % (time.time() - t0))
+
+    t0 = time.time()
+    model.to_device()
+    log("to_cuda (H2D + BF16->FP16 on the device) in %.1f s" % (time.time() - t0))
+    engine = eng_mod.Engine(model, cfg, use_graph=not a.no_graph)
+    prompt = eng_mod.seeded_tokens(a.seed, a.prompt, cfg.vocab)
+
+    # ---- decode: W untimed warm-up steps, then exactly K timed steps ------------------
+    engine.generate(prompt, a.warmup + 1)
+    engine.reset()
+    pkg.capi.sync()
+    w0 = time.time()
+    toks, st = engine.generate(prompt, a.steps + 1)   # prompt pass + K decode steps
+    pkg.capi.sync()
+    wall = time.time() - w0
+    K = st.n_decode_steps
+    assert K == a.steps
+    ms_per_step = st.decode_ms / K
+    tok_s = 1e3 / ms_per_step
+    ctx_avg = a.prompt + (K + 1) / 2.0  # keys attended, averaged over the timed steps
+    frac = decode_bytes(ctx_avg) * tok_s / HBM_PEAK
+    log("decode: %d steps in %.2f ms -> %.1f tok/s (%.1f%% of HBM roofline), prompt pass %.2f ms, wall %.2f s"
+        % (K, st.decode_ms, tok_s, 100 * frac, st.prefill_ms, wall))
+
+    # ---- dominant kernel against its roofline (HIP events on its own stream) -------------
+    roof = kernel_roofline(pkg, model, cfg)
+
+    # ---- 8192-token prompt pass ---------------------------------------------------------------
+    prefill = None
+    if not a.no_prefill_8k:
+        T = 8192
+        p8k = eng_mod.seeded_tokens(a.seed + 1, T, cfg.vocab)
+        engine.reset()
+        engine.generate(p8k, 1)  # warm-up (first use of the large-tile kernels)
+        engine.reset()
+        _, st8 = engine.generate(p8k, 1)
+        sec = st8.prefill_ms * 1e-3
+        prefill = {"tokens": T, "ms": st8.prefill_ms, "tok_per_s": T / sec,
+                   "flops": prefill_flops(T), "mfma_frac": prefill_flops(T) / sec / MFMA_F16_PEAK,
+                   "peak_tflops": MFMA_F16_PEAK / 1e12}
+        log("prefill 8192: %.1f ms -> %.0f tok/s (%.1f%% of fp16 MFMA peak)"
+            % (st8.prefill_ms, T / sec, 100 * prefill["mfma_frac"]))
+        # long-context decode (KV streaming next to weight streaming), 64 steps at ctx ~8.2K
+        engine.reset()
+        _, stl = engine.generate(p8k, 65)
+        ms_l = stl.decode_ms / stl.n_decode_steps
+        prefill["decode_at_8k"] = {"steps": stl.n_decode_steps, "ms_per_step": ms_l, "tok_per_s": 1e3 / ms_l,
+                                   "hbm_frac": decode_bytes(T + 33) * (1e3 / ms_l) / HBM_PEAK}
+        log("decode at ctx 8.2K: %.1f tok/s (%.1f%% of HBM roofline)"
+            % (1e3 / ms_l, 100 * prefill["decode_at_8k"]["hbm_frac"]))
+    engine.close()
+
+    # ---- CPU baseline: fp32 port of the reference forward pass on the host cores ---------------
+    cpu = None
+    if orc is not None:
+        cd = {k: getattr(cfg, k) for k, _ in cfg._fields_}
+        cd["max_pos"] = 256
+        om = orc.Model(cd, orc_w, orc.ORC_FP32)
+        t0 = time.time()
+        tok, _, _ = om.forward(prompt)
+        t_prefill = time.time() - t0
+        t0 = time.time()
+        for _ in range(a.cpu_steps):
+            tok, _, _ = om.forward([tok])
+        t_dec = time.time() - t0
+        cpu = {"value": a.cpu_steps / t_dec, "unit": "tok/s", "cores": orc.num_threads(), "kind": "port",
+               "sample": "%d decode steps after a %d-token prompt on the same seeded LLaMA3-8B weights "
+                         "(fp32 activations and accumulation, fp16 weight values)" % (a.cpu_steps, a.prompt),
+               "prefill_tok_per_s": a.prompt / t_prefill}
+        log("cpu baseline: decode %.2f tok/s, prompt %.1f tok/s on %d threads"
+            % (cpu["value"], cpu["prefill_tok_per_s"], cpu["cores"]))
+        om.close()
+    model.close()
+
+    out = {
+        "metric": "LLaMA3-8B bs1 decode tok/s (% HBM roofline); prefill tok/s at 8K (% MFMA)",
+        "value": tok_s, "unit": "tok/s", "n_gpus": 1, "steps": K, "warmup": a.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "fp16", "data": "synthetic",
+        "config": {"workload": "LLaMA3-8B (32 layers, d 4096, 32/8 heads, FFN 14336, vocab 128256), seeded "
+                               "random-init bf16 weights converted to fp16 at load, batch 1, prompt %d, %d greedy "
+                               "decode steps, fp16 KV cache" % (a.prompt, K),
+                   "prompt_tokens": a.prompt, "decode_steps": K, "graph": not a.no_graph},
+        "decode_hbm_frac": frac, "decode_bytes_per_token": decode_bytes(ctx_avg),
+        "prompt_pass_ms": st.prefill_ms,
+        "roofline": roof, "cpu_baseline": cpu, "prefill_8k": prefill,
+        "first_tokens": [int(t) for t in toks[:8]],
+    }
+    print(json.dumps(out), flush=True)
+
+
+def kernel_roofline(pkg, model, cfg):
+    """Average duration of the fused gate/up SwiGLU GEMV (the kernel that moves
+    most bytes per decode token: 2 x 14336 x 4096 fp16 weights per launch),
+    timed with HIP events on the stream it runs on, cycling through the 32
+    layers' weights so no launch finds its weights in a cache."""
+    lib = pkg.lib()
+    ops = pkg.ops
+    d, F = cfg.d_model, cfg.ffn_dim
+    rng = np.random.default_rng(0)
+    x = pkg.capi.DevBuf.from_host(np.ascontiguousarray(rng.standard_normal(d).astype(np.float16)).view(np.uint16))
+    out = pkg.capi.DevBuf((F,), np.uint16)
+    h = model.handle.contents
+    wg = [h.layers[l].contents.mlp_gate_proj.contents.d_fp16_tensor for l in range(cfg.n_layers)]
+    wu = [h.layers[l].contents.mlp_up_proj.contents.d_fp16_tensor for l in range(cfg.n_layers)]
+    timer = ops.Timer()
+
+    def issue(stream):
+        for l in range(cfg.n_layers):
+            pkg.capi.check(lib.llm_linear_swiglu(x.ptr, d, wg[l], wu[l], out.ptr, F, 1, F, d, stream))
+
+    ms = timer.time(issue, iters=8, warmup=2) / cfg.n_layers
+    alg = 2 * 2 * F * d + 2 * d + 2 * F  # two weight matrices + activation in + result out
+    achieved = alg / (ms * 1e-3)
+    return {"kernel": "gemv_swiglu_kernel (gate+up, N=14336, K=4096, T=1)", "bound": "hbm",
+            "achieved": achieved / 1e9, "peak": HBM_PEAK / 1e9, "unit": "GB/s", "frac": achieved / HBM_PEAK,
+            "traffic": None, "avg_launch_us": ms * 1e3, "algorithmic_bytes_per_launch": alg,
+            "launches_timed": 8 * cfg.n_layers}
+
+
+if __name__ == "__main__":
+    main()

@@ -227,7 +227,7 @@ class DevBuf:
         return out
 
     def zero(self):
-        check(lib().llm_fill_zero(self.ptr, (self.nbytes + 3) // 4 * 4 if self.nbytes % 4 == 0 else self.nbytes, None))
+        check(lib().llm_fill_zero(self.ptr, self.nbytes, None))
         check(lib().llm_device_sync())
 
     def free(self):

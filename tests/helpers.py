@@ -17,9 +17,10 @@ def bits(a):
 
 
 def mixed_err(a_bits, b_bits):
-    """max_i |a-b| / max(1, |b|): absolute below magnitude 1, relative above."""
+    """max_i |a-b| / (1 + |b|).  err <= tol is |a-b| <= tol + tol*|b| for every element, i.e.
+    numpy.allclose(a, b, atol=tol, rtol=tol): the max-abs / rel tolerance with both set to tol."""
     a, b = f16(a_bits), f16(b_bits)
-    return float(np.max(np.abs(a - b) / np.maximum(1.0, np.abs(b)))) if a.size else 0.0
+    return float(np.max(np.abs(a - b) / (1.0 + np.abs(b)))) if a.size else 0.0
 
 
 def ulp_diff(a_bits, b_bits):

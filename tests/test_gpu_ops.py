@@ -1,0 +1,334 @@
+"""GPU parity of every kernel entry point against the CPU oracle on the same
+seeded inputs, through the C-ABI.  Integer/byte work (conversion, gather,
+argmax) is bit-exact; floating-point ops stay inside the 2e-2 max-abs/rel
+tolerance the task states, and tighter bounds are asserted where the kernel
+was built to reproduce the oracle's bits (RMSNorm, RoPE, residual)."""
+import numpy as np
+import pytest
+
+from oracle import pyoracle as orc
+from tests import helpers as H
+
+pytestmark = pytest.mark.gpu
+TOL = H.TOL
+# projections: fp32 accumulation in a different order moves a result by at most one fp16 rounding step
+# (9.8e-4 at magnitude 1..2, relative above), twice that with the residual's second rounding
+TIGHT = 4e-3
+
+
+def say(*a):
+    print(*a, flush=True)
+
+
+# ---- BF16 -> FP16: bit-exact -----------------------------------------------------------------
+def test_convert_all_65536_patterns(gpu):
+    src = np.arange(65536, dtype=np.uint32).astype(np.uint16)
+    assert np.array_equal(gpu.ops.bf16_to_fp16(src), orc.bf16_to_fp16(src))
+
+
+@pytest.mark.parametrize("n", [0, 1, 7, 8, 9, 1000003])
+def test_convert_ragged_sizes(gpu, n):
+    rng = np.random.default_rng(n)
+    src = rng.integers(0, 65536, size=n, dtype=np.uint32).astype(np.uint16)
+    if n == 0:
+        assert gpu.lib().llm_bf16_to_fp16(1, 1, 0, None) == 0
+        return
+    assert np.array_equal(gpu.ops.bf16_to_fp16(src), orc.bf16_to_fp16(src))
+
+
+def test_convert_llama3_8b_ffn_tensor(gpu):
+    # 4096 x 14336 seeded N(0, 0.02) bf16
+    src = gpu.engine.seeded_normal_bf16(42, 7, 4096 * 14336)
+    say("convert 4096x14336")
+    assert np.array_equal(gpu.ops.bf16_to_fp16(src), orc.bf16_to_fp16(src))
+
+
+# ---- embedding: exact ----------------------------------------------------------------------------
+def test_embed_gather_exact_and_bad_id_is_nan(gpu):
+    rng = np.random.default_rng(1)
+    table = H.bits(rng.standard_normal((1000, 4096)))
+    ids = np.array([5, 999, 0, 5, 123], np.int32)
+    assert np.array_equal(gpu.ops.embed_gather(table, ids), orc.embed(table, ids))
+    out = gpu.ops.embed_gather(table, np.array([1000, -1, 3], np.int32))
+    assert np.all(out[:2] == 0x7fff) and np.array_equal(out[2], table[3])
+
+
+# ---- RMSNorm ------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("T,d", [(1, 4096), (128, 4096), (8192, 4096), (3, 256), (2, 512), (2, 16384)])
+def test_rmsnorm(gpu, T, d):
+    rng = np.random.default_rng(T + d)
+    x = H.bits(rng.standard_normal((T, d)))
+    g = H.bits(1.0 + 0.1 * rng.standard_normal(d))
+    say("rmsnorm", T, d)
+    got, want = gpu.ops.rmsnorm(x, g), orc.rmsnorm(x, g)
+    mism = float(np.mean(got != want))
+    say("  mismatching elements:", mism, "max ulp:", int(H.ulp_diff(got, want).max()))
+    assert H.mixed_err(got, want) <= TOL
+    assert np.array_equal(got, want)  # same summation tree, same eps promotion, correctly rounded divide
+    assert np.array_equal(gpu.ops.rmsnorm(x, g, inplace=True), want)
+
+
+def test_rmsnorm_rejects_unsupported_width(gpu):
+    with pytest.raises(gpu.LlmError):
+        gpu.ops.rmsnorm(np.zeros((1, 96), np.uint16), np.zeros(96, np.uint16))
+
+
+def test_add_residual(gpu):
+    rng = np.random.default_rng(3)
+    for n in (8, 4096 * 5, 1001 * 8 + 3):
+        a, b = H.bits(rng.standard_normal(n)), H.bits(rng.standard_normal(n))
+        assert np.array_equal(gpu.ops.add_residual(a, b), orc.add(a, b))
+
+
+# ---- RoPE ------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("T", [1, 128, 8192])
+def test_rope_q_and_k_shapes(gpu, T):
+    rng = np.random.default_rng(T)
+    for heads in (32, 8):
+        x = H.bits(rng.standard_normal((T, heads * 128)))
+        say("rope", T, heads)
+        got, want = gpu.ops.rope(x, heads, 128, 0), orc.rope(x, heads, 128, 0)
+        say("  mismatching elements:", float(np.mean(got != want)))
+        assert H.mixed_err(got, want) <= TOL
+        assert np.array_equal(got, want)  # same libm table, unfused rotate
+
+
+def test_rope_offset_and_small_head(gpu):
+    rng = np.random.default_rng(5)
+    x = H.bits(rng.standard_normal((9, 8 * 32)))
+    assert np.array_equal(gpu.ops.rope(x, 8, 32, 50), orc.rope(x, 8, 32, 50))
+
+
+@pytest.mark.parametrize("T,pos0", [(1, 0), (1, 77), (5, 3), (100, 28)])
+def test_rope_kv_append_layouts(gpu, T, pos0):
+    rng = np.random.default_rng(T * 100 + pos0)
+    Hq, Hkv, hd, max_pos = 8, 2, 32, 128
+    qd, kvd = Hq * hd, Hkv * hd
+    qkv = H.bits(rng.standard_normal((T, qd + 2 * kvd)))
+    q2, kc, vc = gpu.ops.rope_kv_append(qkv, Hq, Hkv, hd, pos0, max_pos)
+    q_want = orc.rope(np.ascontiguousarray(qkv[:, :qd]), Hq, hd, pos0)
+    k_want = orc.rope(np.ascontiguousarray(qkv[:, qd:qd + kvd]), Hkv, hd, pos0)
+    assert np.array_equal(q2[:, :qd], q_want)
+    assert np.array_equal(q2[:, qd:], qkv[:, qd:])  # K and V columns of the buffer are left alone
+    kc_want = np.zeros_like(kc)
+    vc_want = np.zeros_like(vc)
+    kc_want[:, pos0:pos0 + T, :] = k_want.reshape(T, Hkv, hd).transpose(1, 0, 2)
+    vc_want[:, :, pos0:pos0 + T] = qkv[:, qd + kvd:].reshape(T, Hkv, hd).transpose(1, 2, 0)
+    assert np.array_equal(kc, kc_want) and np.array_equal(vc, vc_want)
+
+
+# ---- projections at LLaMA3-8B layer shapes ----------------------------------------------------------------
+SHAPES = {"qkv": (4096, 6144), "o": (4096, 4096), "down": (14336, 4096)}
+
+
+def _proj_inputs(seed, T, K, N):
+    rng = np.random.default_rng(seed)
+    x = H.bits(rng.standard_normal((T, K)))
+    w = H.bits(0.02 * rng.standard_normal((N, K), dtype=np.float32))
+    return x, w
+
+
+@pytest.mark.parametrize("name", list(SHAPES))
+@pytest.mark.parametrize("T", [1, 4, 16])
+def test_linear_skinny(gpu, name, T):
+    K, N = SHAPES[name]
+    x, w = _proj_inputs(T * 7 + K, T, K, N)
+    say("linear", name, T)
+    got, want = gpu.ops.linear(x, w), orc.linear(x, w)
+    e = H.mixed_err(got, want)
+    say("  err", e, "mismatch", float(np.mean(got != want)), "max ulp", int(H.ulp_diff(got, want).max()))
+    assert e <= TIGHT
+
+
+@pytest.mark.parametrize("T", [1, 4, 16])
+def test_linear_residual_epilogue(gpu, T):
+    K, N = 4096, 4096
+    x, w = _proj_inputs(T + 99, T, K, N)
+    res = H.bits(np.random.default_rng(T).standard_normal((T, N)))
+    got = gpu.ops.linear(x, w, residual=res)
+    want = orc.add(orc.linear(x, w), res)
+    assert H.mixed_err(got, want) <= TIGHT
+
+
+@pytest.mark.parametrize("T", [1, 4, 16])
+def test_swiglu_skinny(gpu, T):
+    K, N = 4096, 14336
+    rng = np.random.default_rng(T + 5)
+    x = H.bits(rng.standard_normal((T, K)))
+    wg = H.bits(0.02 * rng.standard_normal((N, K), dtype=np.float32))
+    wu = H.bits(0.02 * rng.standard_normal((N, K), dtype=np.float32))
+    say("swiglu", T)
+    got, want = gpu.ops.linear_swiglu(x, wg, wu), orc.linear_swiglu(x, wg, wu)
+    e = H.mixed_err(got, want)
+    say("  err", e, "max ulp", int(H.ulp_diff(got, want).max()))
+    assert e <= TOL
+
+
+@pytest.mark.parametrize("T,K,N", [(17, 256, 384), (33, 768, 256), (64, 256, 768), (100, 4096, 512),
+                                   (128, 4096, 6144), (200, 512, 1040)])
+def test_linear_gemm_ragged_shapes(gpu, T, K, N):
+    x, w = _proj_inputs(T + K + N, T, K, N)
+    res = H.bits(np.random.default_rng(1).standard_normal((T, N)))
+    say("gemm", T, K, N)
+    got, want = gpu.ops.linear(x, w), orc.linear(x, w)
+    assert got.shape == (T, N)
+    e = H.mixed_err(got, want)
+    say("  err", e, "max ulp", int(H.ulp_diff(got, want).max()))
+    assert e <= TIGHT
+    got_r = gpu.ops.linear(x, w, residual=res)
+    assert H.mixed_err(got_r, orc.add(orc.linear(x, w), res)) <= TOL
+
+
+def test_linear_gemm_reference_test_operand_pattern(gpu):
+    # the operand pattern of the reference's tests/gemm.cu scaled to a shape the kernels take:
+    # x[i][j] = (i*K + j) % 5 - 2, w likewise; exact in fp32, so any layout slip shows
+    T, K, N = 40, 128, 64
+    x = ((np.arange(T * K).reshape(T, K) % 5) - 2).astype(np.float64)
+    w = ((np.arange(N * K).reshape(N, K) % 7) - 3).astype(np.float64)
+    got = gpu.ops.linear(H.bits(x), H.bits(w))
+    assert np.array_equal(got, H.bits(x @ w.T))
+    assert np.array_equal(gpu.ops.linear(H.bits(x[:1]), H.bits(w)), H.bits(x[:1] @ w.T))
+    assert np.array_equal(gpu.ops.linear(H.bits(x[:5]), H.bits(w)), H.bits(x[:5] @ w.T))
+
+
+@pytest.mark.parametrize("name", list(SHAPES))
+def test_linear_mfma_512(gpu, name):
+    K, N = SHAPES[name]
+    x, w = _proj_inputs(512 + K, 512, K, N)
+    say("mfma 512", name)
+    got, want = gpu.ops.linear(x, w), orc.linear(x, w)
+    e = H.mixed_err(got, want)
+    say("  err", e, "max ulp", int(H.ulp_diff(got, want).max()))
+    assert e <= TIGHT
+
+
+def test_swiglu_mfma_512(gpu):
+    K, N, T = 4096, 14336, 512
+    rng = np.random.default_rng(8)
+    x = H.bits(rng.standard_normal((T, K)))
+    wg = H.bits(0.02 * rng.standard_normal((N, K), dtype=np.float32))
+    wu = H.bits(0.02 * rng.standard_normal((N, K), dtype=np.float32))
+    got, want = gpu.ops.linear_swiglu(x, wg, wu), orc.linear_swiglu(x, wg, wu)
+    e = H.mixed_err(got, want)
+    say("swiglu 512 err", e)
+    assert e <= TOL
+
+
+def test_linear_mfma_8192_rows_sampled(gpu):
+    # full T = 8192 on the GPU; the oracle follows 96 of the rows (rows are independent)
+    K, N, T = 4096, 6144, 8192
+    x, w = _proj_inputs(77, T, K, N)
+    got = gpu.ops.linear(x, w)
+    rows = np.r_[0:32, 4080:4112, 8160:8192]
+    want = orc.linear(np.ascontiguousarray(x[rows]), w)
+    e = H.mixed_err(got[rows], want)
+    say("mfma 8192 err", e)
+    assert e <= TIGHT
+    # linearity in x at full size: doubling x doubles every fp32 sum exactly
+    # (outputs that round into the fp16 subnormal range lose the doubled bit: left out)
+    x2 = H.bits(2.0 * H.f16(x))
+    a, b = H.f16(gpu.ops.linear(x2, w)), 2.0 * H.f16(got)
+    normal = np.abs(b) >= 2.0 ** -12
+    assert np.array_equal(a[normal], b[normal])
+
+
+# ---- LM head + argmax -----------------------------------------------------------------------------------------
+def test_lmhead_argmax_full_vocab(gpu):
+    K, V = 4096, 128256
+    rng = np.random.default_rng(9)
+    x = H.bits(rng.standard_normal((1, K)))
+    w = H.bits(0.02 * rng.standard_normal((V, K), dtype=np.float32))
+    say("lm head")
+    tok, logits = gpu.ops.lmhead_argmax(x, w)
+    want = orc.linear(x, w).reshape(-1)
+    e = H.mixed_err(logits, want)
+    say("  err", e, "token", tok, orc.argmax_f16(want))
+    assert e <= TIGHT
+    assert tok == orc.argmax_f16(logits)  # argmax over the kernel's own fp16 logits: exact
+
+
+def test_argmax_ties_zero_signs_nan(gpu):
+    b = H.bits
+    cases = [b([1.0, 3.0, 3.0, 2.0]), b([-0.0, 0.0, -1.0]), b([0.0, -0.0]), b([-np.inf, -5.0]),
+             np.array([0x7e00, 0xfe00], np.uint16), np.array([0x3c00, 0x7e00, 0x3800], np.uint16)]
+    rng = np.random.default_rng(10)
+    big = b(rng.standard_normal(128256))
+    big[[77, 90000]] = big.view(np.float16).max().view(np.uint16)  # a tie far apart: lowest index wins
+    cases.append(big)
+    cases.append(b(np.round(rng.standard_normal(300000) * 4) / 4))  # many ties
+    for c in cases:
+        assert gpu.ops.argmax_f16(c) == orc.argmax_f16(c)
+
+
+# ---- attention ----------------------------------------------------------------------------------------------------
+def _attn_inputs(seed, P, Hq, Hkv, hd):
+    rng = np.random.default_rng(seed)
+    return (H.bits(rng.standard_normal((P, Hq * hd))), H.bits(rng.standard_normal((P, Hkv * hd))),
+            H.bits(rng.standard_normal((P, Hkv * hd))))
+
+
+@pytest.mark.parametrize("ctx,max_pos", [(1, 64), (2, 64), (63, 64), (64, 64), (65, 2048), (384, 2048),
+                                         (2048, 2048), (8448, 8704), (8704, 8704)])
+def test_attn_decode_llama3_8b_heads(gpu, ctx, max_pos):
+    Hq, Hkv, hd = 32, 8, 128
+    q, k, v = _attn_inputs(ctx, ctx, Hq, Hkv, hd)
+    kc, vc = gpu.ops.kv_layout(k, v, Hkv, hd, max_pos)
+    # rows past ctx hold stale junk from an earlier, longer sequence
+    kc[:, ctx:, :] = H.bits(np.float16(3.0))
+    vc[:, :, ctx:] = H.bits(np.float16(-7.0))
+    say("attn decode", ctx, max_pos)
+    got = gpu.ops.attn_decode(q[-1], kc, vc, ctx, Hq, Hkv, hd, repeats=2)
+    want = orc.attention(q[-1:], k, v, ctx - 1, Hq, Hkv, hd).reshape(-1)
+    e = H.mixed_err(got, want)
+    say("  err", e, "max ulp", int(H.ulp_diff(got, want).max()))
+    assert e <= TOL
+
+
+def test_attn_decode_small_heads_and_gqa_map(gpu):
+    Hq, Hkv, hd, ctx = 8, 2, 32, 20
+    q, k, v = _attn_inputs(3, ctx, Hq, Hkv, hd)
+    # V rows constant per KV head: the output reveals which KV head each query head read
+    v = H.bits(np.repeat(np.arange(1, Hkv + 1, dtype=np.float64)[None, :], ctx, 0).repeat(hd, 1))
+    kc, vc = gpu.ops.kv_layout(k, v, Hkv, hd, 64)
+    got = H.f16(gpu.ops.attn_decode(q[-1], kc, vc, ctx, Hq, Hkv, hd)).reshape(Hq, hd)
+    for h in range(Hq):
+        assert np.allclose(got[h], h // 4 + 1, atol=2e-3)
+
+
+@pytest.mark.parametrize("T,pos0,Hq,Hkv,hd", [(1, 0, 8, 2, 32), (16, 0, 8, 2, 32), (33, 7, 8, 2, 32),
+                                              (64, 0, 32, 8, 128), (100, 60, 32, 8, 128), (512, 0, 32, 8, 128)])
+def test_attn_prefill(gpu, T, pos0, Hq, Hkv, hd):
+    P = pos0 + T
+    q, k, v = _attn_inputs(T + pos0, P, Hq, Hkv, hd)
+    max_pos = (P + 63) // 64 * 64
+    kc, vc = gpu.ops.kv_layout(k, v, Hkv, hd, max_pos)
+    say("attn prefill", T, pos0, Hq, hd)
+    got = gpu.ops.attn_prefill(q[pos0:], kc, vc, pos0, Hq, Hkv, hd)
+    want = orc.attention(np.ascontiguousarray(q[pos0:]), k, v, pos0, Hq, Hkv, hd)
+    e = H.mixed_err(got, want)
+    say("  err", e, "max ulp", int(H.ulp_diff(got, want).max()))
+    assert e <= TOL
+
+
+def test_attn_prefill_8192_last_rows_and_uniform_key_property(gpu):
+    T, Hq, Hkv, hd = 8192, 32, 8, 128
+    q, k, v = _attn_inputs(11, T, Hq, Hkv, hd)
+    kc, vc = gpu.ops.kv_layout(k, v, Hkv, hd, T)
+    say("attn prefill 8192")
+    got = gpu.ops.attn_prefill(q, kc, vc, 0, Hq, Hkv, hd)
+    # oracle on the first rows and on a late chunk
+    want0 = orc.attention(np.ascontiguousarray(q[:64]), k, v, 0, Hq, Hkv, hd)
+    assert H.mixed_err(got[:64], want0) <= TOL
+    want1 = orc.attention(np.ascontiguousarray(q[8128:8160]), k, v, 8128, Hq, Hkv, hd)
+    e = H.mixed_err(got[8128:8160], want1)
+    say("  late rows err", e)
+    assert e <= TOL
+    # size-independent property: identical keys => row i is the mean of V[0..i]
+    k1 = np.tile(k[:1], (T, 1))
+    kc1, _ = gpu.ops.kv_layout(k1, v, Hkv, hd, T)
+    out = H.f16(gpu.ops.attn_prefill(q, kc1, vc, 0, Hq, Hkv, hd))
+    vf = H.f16(v)
+    csum = np.cumsum(vf, axis=0) / np.arange(1, T + 1)[:, None]
+    for h in (0, 5, 31):
+        kv = h // 4
+        assert np.allclose(out[:, h * hd:(h + 1) * hd], csum[:, kv * hd:(kv + 1) * hd], atol=5e-3)
