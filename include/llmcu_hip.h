@@ -130,6 +130,17 @@ int llm_linear_swiglu(const uint16_t *x_dev, int ldx, const uint16_t *wgate_dev,
                       const uint16_t *wup_dev, uint16_t *out_dev, int ldo, int T, int N, int K,
                       llm_stream_t stream);
 
+/* One-row projections with the RMSNorm of the input folded in (the decode
+ * step): out = linear(rmsnorm(x, gain, eps), w).  Replaces compute_layer_norm
+ * followed by compute_qkv_tensors, resp. by the gate/up launch of
+ * compute_feedforward (src/inference/inference.cu:160-163,179-182) for T = 1;
+ * same bits as llm_rmsnorm followed by llm_linear / llm_linear_swiglu. */
+int llm_norm_linear(const uint16_t *x_dev, const uint16_t *gain_dev, double eps, const uint16_t *w_dev,
+                    uint16_t *out_dev, int N, int K, llm_stream_t stream);
+int llm_norm_linear_swiglu(const uint16_t *x_dev, const uint16_t *gain_dev, double eps,
+                           const uint16_t *wgate_dev, const uint16_t *wup_dev, uint16_t *out_dev, int N,
+                           int K, llm_stream_t stream);
+
 /* ---- attention ------------------------------------------------------------------ */
 /* Replaces compute_attention and its three kernels
  * (src/inference/inference.cu:698-947) for one new row: causal GQA attention
@@ -145,6 +156,15 @@ int llm_attn_decode(const uint16_t *q_dev, const uint16_t *k_cache_dev, const ui
                     uint16_t *out_dev, int ctx_host, const int32_t *ctx_dev, int n_heads,
                     int n_kv_heads, int head_dim, int max_pos, void *workspace_dev,
                     llm_stream_t stream);
+/* The decode step's form: takes the raw projection row qkv ([(Hq+2Hkv)*hd],
+ * not rotated), applies RoPE for position pos = pos_host + (pos_dev ? *pos_dev : 0)
+ * to Q and K, appends K and V to the caches at that position, and attends over
+ * rows 0..pos.  One launch for rope_scaling + compute_attention
+ * (src/inference/inference.cu:621-734).  qkv is left unmodified. */
+int llm_attn_decode_rope(const uint16_t *qkv_dev, uint16_t *k_cache_dev, uint16_t *v_cache_dev,
+                         uint16_t *out_dev, int pos_host, const int32_t *pos_dev, const float *table_dev,
+                         int n_heads, int n_kv_heads, int head_dim, int max_pos, void *workspace_dev,
+                         llm_stream_t stream);
 /* Same attention for T query rows at positions pos0..pos0+T-1 (prompt pass),
  * streaming softmax on MFMA tiles; never materialises [H,T,T].
  * q: [T, ldq] with head h at columns h*hd; out: [T, ldo].  Cache rows beyond
@@ -166,7 +186,12 @@ size_t llm_lmhead_workspace_bytes(int vocab);
 int llm_lmhead_argmax(const uint16_t *x_dev, const uint16_t *w_dev, uint16_t *logits_dev,
                       int32_t *token_dev, int32_t *tokens_dev, int32_t *pos_dev, int vocab, int K,
                       void *workspace_dev, llm_stream_t stream);
-/* argmax alone over fp16 values (same tie/NaN rule). */
+/* Same with the final RMSNorm of x folded in (compute_layer_norm(model->norm)
+ * + compute_lm_head, src/inference/inference.cu:188-190). */
+int llm_norm_lmhead_argmax(const uint16_t *x_dev, const uint16_t *gain_dev, double eps, const uint16_t *w_dev,
+                           uint16_t *logits_dev, int32_t *token_dev, int32_t *tokens_dev, int32_t *pos_dev,
+                           int vocab, int K, void *workspace_dev, llm_stream_t stream);
+/* argmax alone over fp16 values (same tie/NaN rule); workspace as for the LM head of n rows. */
 int llm_argmax_f16(const uint16_t *logits_dev, int n, int32_t *token_dev, void *workspace_dev,
                    llm_stream_t stream);
 

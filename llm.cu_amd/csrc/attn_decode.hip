@@ -1,95 +1,160 @@
-// Causal GQA attention for one new token over the fp16 KV cache.
+// Causal GQA attention for one new token over the fp16 KV cache, optionally
+// with RoPE and the KV-cache append of that token folded in.
 //
 // Cache layout (per layer), chosen so that both passes stream contiguous
 // memory per KV head:
 //   K: [Hkv][max_pos][hd]   a position's hd values are contiguous  (scores = K . q)
 //   V: [Hkv][hd][max_pos]   a dim's positions are contiguous       (out = V^T-rows . p)
 //
-// Grid (Hkv, splits): a workgroup owns one KV head and one span of positions
-// and serves all G = Hq/Hkv query heads of the group, so each K/V byte is read
-// once.  Per span: scores -> LDS, local max/sum, unnormalised P.V.  The last
-// workgroup of a head to finish (a self-resetting counter) merges the spans.
-// Scores, softmax and P.V stay in fp32 as in the reference
-// (src/inference/inference.cu:736-947); only the final output is rounded.
+// Grid (Hkv, y): a workgroup owns one KV head and serves all G = Hq/Hkv query
+// heads of the group.  Up to 512 keys there is one span of positions: four
+// workgroups per head each take a quarter of the head's dims (each recomputes
+// the cheap scores, so none waits for another) and write the result directly.
+// Beyond that workgroup y takes the 512-position span y with all dims, leaves
+// (max, sum, unnormalised P.V), and the last workgroup of the head to finish
+// (a self-resetting counter) merges the spans.  Scores, softmax and P.V
+// stay in fp32 as in the reference (src/inference/inference.cu:736-947); only
+// the final output is rounded.
 #include <cfloat>
 #include <cmath>
 
 #include "common.hpp"
 
-#define AD_THREADS 256
+#define AD_THREADS 512
+#define AD_WAVES 8
 #define AD_MAX_SPLITS 256
+#define AD_LS 512 // positions per span (longest)
 
-struct AdShape {
-    int splits;
-    int ls_max; // longest span, multiple of 64
+struct AdArgs {
+    const half_t *q;   // plain: rotated queries [Hq*hd]; fused: the raw qkv row [(Hq+2Hkv)*hd]
+    half_t *kc, *vc;   // caches of this layer
+    half_t *out;       // [Hq*hd]
+    const float *table; // fused: (cos, sin) table [max_pos][hd/2][2]
+    int pos_host;
+    const int32_t *pos_dev; // position of the new token = pos_host + *pos_dev; ctx = position + 1
+    int n_kv_heads, max_pos, splits;
+    float *ws_acc, *ws_ml;
+    int *counters;
 };
 
-static AdShape ad_shape(int max_pos, int G) {
-    AdShape s;
-    s.splits = (max_pos + 255) / 256;
-    if (s.splits < 1) s.splits = 1;
-    if (s.splits > 32) s.splits = 32;
-    for (;;) {
-        int per = (max_pos + s.splits - 1) / s.splits;
-        s.ls_max = (per + 63) / 64 * 64;
-        if ((size_t)G * s.ls_max * sizeof(float) <= 40 * 1024 || s.splits >= AD_MAX_SPLITS) break;
-        s.splits *= 2;
-        if (s.splits > AD_MAX_SPLITS) s.splits = AD_MAX_SPLITS;
-    }
-    return s;
-}
+// Every K and V load of the span is issued before anything else (a span is at
+// most 512 positions: 16 + 16 loads of 16 bytes per thread at hd 128), so the
+// whole span costs one trip to HBM instead of one per loop iteration.  In the
+// fused form the new token's own K and V come from the projection row through
+// LDS (and are written to the cache for later steps), so nothing waits on
+// that write.
+//
+// NDIM is the number of head dims this workgroup produces, LS the span length.
+template <int HD, int G, bool FUSED, int NDIM, int LS>
+__device__ __forceinline__ void attn_decode_body(const AdArgs &a, float *sc, half_t *qs, half_t *knew, half_t *vnew,
+                                                 float *s_m, float *s_l, int *s_last, const int pos,
+                                                 const int n_active, const int split, const int d_begin,
+                                                 const bool appender) {
+    constexpr int LPP = HD / 8;                    // lanes per position in the score pass
+    constexpr int PPW = 64 / LPP;                  // positions per wavefront pass
+    constexpr int KIT = LS / (AD_WAVES * PPW);  // K loads per thread
+    constexpr int DPW = NDIM / AD_WAVES;           // dims per wavefront in the P.V pass
+    static_assert(DPW >= 1, "too few dims for the workgroup");
+    constexpr int RR = DPW < 8 ? DPW : 8;          // dim rows per pass
+    constexpr int JL = 64 / RR;                    // lanes along positions (8, 16, 32 or 64)
+    constexpr int VP = DPW / RR;                   // passes over dims
+    constexpr int VIT = LS / (JL * 8);          // V loads per thread and pass
+    constexpr int HALF = HD / 2;
 
-template <int HD, int G>
-__global__ __launch_bounds__(AD_THREADS) void attn_decode_kernel(
-    const half_t *__restrict__ q, const half_t *__restrict__ kc, const half_t *__restrict__ vc,
-    half_t *__restrict__ out, int ctx_host, const int32_t *__restrict__ ctx_dev, int max_pos, int splits,
-    int ls_max, float *__restrict__ ws_acc, float *__restrict__ ws_ml, int *__restrict__ counters) {
-    constexpr int LPP = HD / 8;   // lanes per position in the score pass
-    constexpr int PPW = 64 / LPP; // positions per wavefront pass
-    extern __shared__ float sc[]; // [G][ls_max]
-    __shared__ float s_m[G], s_l[G];
-    __shared__ int s_last;
-
-    const int kvh = blockIdx.x, split = blockIdx.y;
+    const int kvh = blockIdx.x, splits = a.splits;
     const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
-    int ctx = ctx_host + (ctx_dev ? *ctx_dev : 0);
-    if (ctx > max_pos) ctx = max_pos;
-    if (ctx < 1) ctx = 1;
-    const int per = (ctx + splits - 1) / splits;
-    const int ls = (per + 63) / 64 * 64;
-    const int n_active = (ctx + ls - 1) / ls;
-    if (split >= n_active) return;
-    const int s0 = split * ls;
-    const int s1 = ctx < s0 + ls ? ctx : s0 + ls;
-    const int len = s1 - s0;
+    const int max_pos = a.max_pos;
+    const int ctx = pos + 1;
+    const int s0 = split * LS;
+    const int len = ctx - s0 < LS ? ctx - s0 : LS;
     const int len_pad = (len + 63) / 64 * 64;
+    half_t *kbase = a.kc + (size_t)kvh * max_pos * HD;
+    half_t *vrow0 = a.vc + (size_t)kvh * HD * max_pos;
+    const int lpos = pos - s0; // the new token inside this span (last span only)
 
-    // ---- scores ------------------------------------------------------------
+    // ---- 1. all K and V loads of the span ----------------------------------------
     const int sub = lane % LPP;
-    half8_t qreg[G];
+    half8_t kreg[KIT];
 #pragma unroll
-    for (int h = 0; h < G; ++h) qreg[h] = load8(q + (size_t)(kvh * G + h) * HD + sub * 8);
-    const float den = sqrtf((float)HD);
-    const half_t *kbase = kc + (size_t)kvh * max_pos * HD;
-    for (int j = s0 + wave * PPW + lane / LPP; j < s1; j += 4 * PPW) {
-        half8_t kv = load8(kbase + (size_t)j * HD + sub * 8);
-        float part[G];
+    for (int it = 0; it < KIT; ++it) {
+        const int j = it * (AD_WAVES * PPW) + wave * PPW + lane / LPP;
+        kreg[it] = j < len ? load8(kbase + (size_t)(s0 + j) * HD + sub * 8) : half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+    }
+    const int rr = lane / JL, jc = lane % JL;
+    half8_t vreg[VP][VIT];
 #pragma unroll
-        for (int h = 0; h < G; ++h) {
-            part[h] = dot8(kv, qreg[h], 0.f);
+    for (int p = 0; p < VP; ++p) {
+        const int d = d_begin + wave * DPW + p * RR + rr;
 #pragma unroll
-            for (int off = LPP / 2; off >= 1; off >>= 1) part[h] += __shfl_xor(part[h], off);
+        for (int it = 0; it < VIT; ++it) {
+            const int j = (jc + JL * it) * 8;
+            vreg[p][it] = j < len ? load8(vrow0 + (size_t)d * max_pos + s0 + j) : half8_t{0, 0, 0, 0, 0, 0, 0, 0};
         }
-        if (sub == 0) {
+    }
+
+    // ---- 2. queries into LDS; fused: rotate them and the new K, append K/V ---------
+    if (FUSED) {
+        const int Hq = a.n_kv_heads * G;
+        const half_t *qkv = a.q;
+        const float *cs = a.table + (size_t)pos * HALF * 2;
+        for (int p = tid; p < (G + 1) * HALF; p += AD_THREADS) {
+            const int h = p / HALF, i = p % HALF; // h == G: the new key
+            const half_t *src = h < G ? qkv + (size_t)(kvh * G + h) * HD + 2 * i
+                                      : qkv + (size_t)Hq * HD + (size_t)kvh * HD + 2 * i;
+            const float c = cs[2 * i], sn = cs[2 * i + 1];
+            const float e = (float)src[0], o = (float)src[1];
+            const float ce = c * e, so = sn * o, se = sn * e, co = c * o;
+            const half_t re = (half_t)(ce - so), ro = (half_t)(se + co);
+            if (h < G) {
+                qs[h * HD + 2 * i] = re;
+                qs[h * HD + 2 * i + 1] = ro;
+            } else {
+                knew[2 * i] = re;
+                knew[2 * i + 1] = ro;
+                if (appender) {
+                    kbase[(size_t)pos * HD + 2 * i] = re;
+                    kbase[(size_t)pos * HD + 2 * i + 1] = ro;
+                }
+            }
+        }
+        const half_t *vsrc = qkv + (size_t)(Hq + a.n_kv_heads) * HD + (size_t)kvh * HD;
+        for (int d = tid; d < HD; d += AD_THREADS) {
+            const half_t v = vsrc[d];
+            vnew[d] = v;
+            if (appender) vrow0[(size_t)d * max_pos + pos] = v;
+        }
+    } else {
+        for (int c = tid * 8; c < G * HD; c += AD_THREADS * 8) store8(qs + c, load8(a.q + (size_t)kvh * G * HD + c));
+    }
+    __syncthreads();
+
+    // ---- 3. scores ---------------------------------------------------------------------
+    {
+        half8_t qreg[G];
 #pragma unroll
-            for (int h = 0; h < G; ++h) sc[h * ls_max + (j - s0)] = part[h] / den;
+        for (int h = 0; h < G; ++h) qreg[h] = load8(qs + h * HD + sub * 8);
+        const float scale = 1.0f / sqrtf((float)HD);
+#pragma unroll
+        for (int it = 0; it < KIT; ++it) {
+            if (it * (AD_WAVES * PPW) + wave * PPW < len) { // wave-uniform: skip passes beyond the span
+                const int j = it * (AD_WAVES * PPW) + wave * PPW + lane / LPP;
+                half8_t kv = kreg[it];
+                if (FUSED && j == lpos) kv = load8(knew + sub * 8);
+                float part[G];
+#pragma unroll
+                for (int h = 0; h < G; ++h) part[h] = group_sum<LPP>(dot8(kv, qreg[h], 0.f));
+                if (sub == 0 && j < len) {
+#pragma unroll
+                    for (int h = 0; h < G; ++h) sc[h * LS + j] = part[h] * scale;
+                }
+            }
         }
     }
     __syncthreads();
 
-    // ---- local softmax statistics: wavefront w takes heads w, w+4, ... -------
-    for (int h = wave; h < G; h += 4) {
-        float *row = sc + h * ls_max;
+    // ---- 4. local softmax statistics: wavefront w takes heads w, w+8, ... ------------------
+    for (int h = wave; h < G; h += AD_WAVES) {
+        float *row = sc + h * LS;
         float mx = -FLT_MAX;
         for (int j = lane; j < len; j += 64) mx = fmaxf(mx, row[j]);
         mx = wave_max(mx);
@@ -107,85 +172,171 @@ __global__ __launch_bounds__(AD_THREADS) void attn_decode_kernel(
     }
     __syncthreads();
 
-    // ---- unnormalised P.V: wavefront w takes dims [w*HD/4, (w+1)*HD/4) --------
-    {
-        const int rr = lane / 8, jc = lane % 8;
-        const half_t *vbase = vc + (size_t)kvh * HD * max_pos + s0;
-        for (int d0 = wave * (HD / 4); d0 < (wave + 1) * (HD / 4); d0 += 8) {
-            const int d = d0 + rr;
-            float acc[G];
+    // ---- 5. unnormalised P.V from the registers ----------------------------------------------
 #pragma unroll
-            for (int h = 0; h < G; ++h) acc[h] = 0.f;
-            for (int j = jc * 8; j < len; j += 64) {
-                half8_t vv = load8(vbase + (size_t)d * max_pos + j);
+    for (int p = 0; p < VP; ++p) {
+        const int d = d_begin + wave * DPW + p * RR + rr;
+        float acc[G];
+#pragma unroll
+        for (int h = 0; h < G; ++h) acc[h] = 0.f;
+#pragma unroll
+        for (int it = 0; it < VIT; ++it) {
+            const int j = (jc + JL * it) * 8;
+            if (j < len) {
                 float vf[8];
 #pragma unroll
-                for (int i = 0; i < 8; ++i) vf[i] = (j + i < len) ? (float)vv[i] : 0.f;
+                for (int i = 0; i < 8; ++i) vf[i] = (float)vreg[p][it][i];
+                if (FUSED && lpos >= j && lpos < j + 8) { // the chunk that holds the new token (rare)
+                    const float vn = (float)vnew[d];
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) vf[i] = (j + i == lpos) ? vn : vf[i];
+                }
+                if (j + 8 > len) { // the chunk that straddles the end of the span (rare)
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) vf[i] = (j + i < len) ? vf[i] : 0.f;
+                }
 #pragma unroll
                 for (int h = 0; h < G; ++h) {
-                    const float *e = sc + h * ls_max + j;
+                    const float *e = sc + h * LS + j;
 #pragma unroll
                     for (int i = 0; i < 8; ++i) acc[h] = fmaf(e[i], vf[i], acc[h]);
                 }
             }
+        }
 #pragma unroll
-            for (int h = 0; h < G; ++h) {
-#pragma unroll
-                for (int off = 4; off >= 1; off >>= 1) acc[h] += __shfl_xor(acc[h], off);
+        for (int h = 0; h < G; ++h) {
+            if (JL <= 16) {
+                acc[h] = group_sum<(JL <= 16 ? JL : 16)>(acc[h]);
+            } else {
+                acc[h] = group_sum<16>(acc[h]);
+                acc[h] += __shfl_xor(acc[h], 16);
+                if (JL == 64) acc[h] += __shfl_xor(acc[h], 32);
             }
-            if (jc == 0) {
+        }
+        if (jc == 0) {
+            if (n_active == 1) {
 #pragma unroll
-                for (int h = 0; h < G; ++h)
-                    ws_acc[(((size_t)kvh * splits + split) * G + h) * HD + d] = acc[h];
+                for (int h = 0; h < G; ++h) a.out[(size_t)(kvh * G + h) * HD + d] = (half_t)(acc[h] / s_l[h]);
+            } else {
+#pragma unroll
+                for (int h = 0; h < G; ++h) a.ws_acc[(((size_t)kvh * splits + split) * G + h) * HD + d] = acc[h];
             }
         }
     }
+    if (n_active == 1) return;
     if (tid < G) {
-        ws_ml[(((size_t)kvh * splits + split) * G + tid) * 2 + 0] = s_m[tid];
-        ws_ml[(((size_t)kvh * splits + split) * G + tid) * 2 + 1] = s_l[tid];
+        a.ws_ml[(((size_t)kvh * splits + split) * G + tid) * 2 + 0] = s_m[tid];
+        a.ws_ml[(((size_t)kvh * splits + split) * G + tid) * 2 + 1] = s_l[tid];
     }
 
-    // ---- the last workgroup of this head merges the spans --------------------
+    // ---- 6. the last workgroup of this head merges the spans ------------------------------------
     __threadfence();
     __syncthreads();
     if (tid == 0) {
-        int old = atomicAdd(&counters[kvh], 1);
-        s_last = (old == n_active - 1);
+        int old = atomicAdd(&a.counters[kvh], 1);
+        *s_last = (old == n_active - 1);
     }
     __syncthreads();
-    if (!s_last) return;
+    if (!*s_last) return;
     __threadfence();
+    // (max, sum) of every span into LDS (reusing the score buffer) in one round of
+    // independent loads, then per-span weights exp(m_s - M), then a weighted sum
+    // whose loads do not depend on one another
+    float *wgt = sc;                 // [n_active][G]: m_s, then the weights
+    float *lsum = sc + n_active * G; // [n_active][G]: l_s
+    for (int idx = tid; idx < n_active * G; idx += AD_THREADS) {
+        const size_t b = ((size_t)kvh * splits + idx / G) * G + idx % G;
+        wgt[idx] = a.ws_ml[b * 2];
+        lsum[idx] = a.ws_ml[b * 2 + 1];
+    }
+    __syncthreads();
+    if (tid < G) {
+        float M = -FLT_MAX;
+        for (int s = 0; s < n_active; ++s) M = fmaxf(M, wgt[s * G + tid]);
+        float L = 0.f;
+        for (int s = 0; s < n_active; ++s) {
+            const float w = expf(wgt[s * G + tid] - M);
+            wgt[s * G + tid] = w;
+            L += lsum[s * G + tid] * w;
+        }
+        s_l[tid] = L;
+    }
+    __syncthreads();
     for (int idx = tid; idx < G * HD; idx += AD_THREADS) {
         const int h = idx / HD, d = idx % HD;
-        float M = -FLT_MAX;
-        for (int s = 0; s < n_active; ++s)
-            M = fmaxf(M, ws_ml[(((size_t)kvh * splits + s) * G + h) * 2]);
-        float L = 0.f, o = 0.f;
-        for (int s = 0; s < n_active; ++s) {
-            const size_t b = ((size_t)kvh * splits + s) * G + h;
-            const float wgt = expf(ws_ml[b * 2] - M);
-            L += ws_ml[b * 2 + 1] * wgt;
-            o += ws_acc[b * HD + d] * wgt;
+        float o = 0.f;
+        int s = 0;
+        for (; s + 8 <= n_active; s += 8) {
+            float v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) v[u] = a.ws_acc[(((size_t)kvh * splits + s + u) * G + h) * HD + d];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) o += v[u] * wgt[(s + u) * G + h];
         }
-        out[(size_t)(kvh * G + h) * HD + d] = (half_t)(o / L);
+        for (; s < n_active; ++s) o += a.ws_acc[(((size_t)kvh * splits + s) * G + h) * HD + d] * wgt[s * G + h];
+        a.out[(size_t)(kvh * G + h) * HD + d] = (half_t)(o / s_l[h]);
     }
-    if (tid == 0) counters[kvh] = 0; // ready for the next launch
+    if (tid == 0) a.counters[kvh] = 0; // ready for the next launch
 }
 
-template <int HD, int G>
-static int launch_decode(const half_t *q, const half_t *kc, const half_t *vc, half_t *out, int ctx_host,
-                         const int32_t *ctx_dev, int n_kv_heads, int max_pos, void *ws, hipStream_t s) {
-    const AdShape sh = ad_shape(max_pos, G);
-    const int Hq = n_kv_heads * G;
-    float *ws_acc = (float *)ws;
-    float *ws_ml = ws_acc + (size_t)Hq * AD_MAX_SPLITS * HD;
-    int *counters = (int *)(ws_ml + (size_t)Hq * AD_MAX_SPLITS * 2);
-    const size_t smem = (size_t)G * sh.ls_max * sizeof(float);
-    LLM_REQUIRE(smem <= 64 * 1024, "llm_attn_decode: max_pos=%d needs %zu bytes of LDS", max_pos, smem);
-    attn_decode_kernel<HD, G><<<dim3(n_kv_heads, sh.splits), dim3(AD_THREADS), smem, s>>>(
-        q, kc, vc, out, ctx_host, ctx_dev, max_pos, sh.splits, sh.ls_max, ws_acc, ws_ml, counters);
+template <int HD, int G, bool FUSED, int DSN>
+__global__ __launch_bounds__(AD_THREADS) void attn_decode_kernel(const AdArgs a) {
+    __shared__ float sc[G * AD_LS];
+    __shared__ __attribute__((aligned(16))) half_t qs[G * HD];
+    __shared__ __attribute__((aligned(16))) half_t knew[HD];
+    __shared__ __attribute__((aligned(16))) half_t vnew[HD];
+    __shared__ float s_m[G], s_l[G];
+    __shared__ int s_last;
+    int pos = a.pos_host + (a.pos_dev ? *a.pos_dev : 0);
+    if (pos > a.max_pos - 1) pos = a.max_pos - 1;
+    if (pos < 0) pos = 0;
+    const int n_active = pos / AD_LS + 1;
+    const int y = blockIdx.y;
+    if (n_active == 1) {
+        // one span: workgroups 0..DSN-1 of the head each take a slice of its dims and write
+        // the result directly (no synchronisation between them)
+        if (y >= DSN) return;
+        attn_decode_body<HD, G, FUSED, HD / DSN, AD_LS>(a, sc, qs, knew, vnew, s_m, s_l, &s_last, pos, 1, 0,
+                                                        y * (HD / DSN), y == 0);
+    } else {
+        // several spans: workgroup y takes span y with all dims; the last to finish merges
+        if (y >= n_active) return;
+        attn_decode_body<HD, G, FUSED, HD, AD_LS>(a, sc, qs, knew, vnew, s_m, s_l, &s_last, pos, n_active, y, 0,
+                                                  y == n_active - 1);
+    }
+}
+
+template <int HD, int G, bool FUSED>
+static int launch_decode(AdArgs a, void *ws, hipStream_t s) {
+    constexpr int DSN = HD >= 128 ? 4 : 1;
+    const int Hq = a.n_kv_heads * G;
+    a.ws_acc = (float *)ws;
+    a.ws_ml = a.ws_acc + (size_t)Hq * AD_MAX_SPLITS * HD;
+    a.counters = (int *)(a.ws_ml + (size_t)Hq * AD_MAX_SPLITS * 2);
+    const int splits = (a.max_pos + AD_LS - 1) / AD_LS;
+    LLM_REQUIRE(splits <= AD_MAX_SPLITS, "llm_attn_decode: max_pos=%d exceeds %d", a.max_pos, AD_MAX_SPLITS * AD_LS);
+    a.splits = splits;
+    const int gy = splits > DSN ? splits : DSN;
+    attn_decode_kernel<HD, G, FUSED, DSN><<<dim3(a.n_kv_heads, gy), dim3(AD_THREADS), 0, s>>>(a);
     LLM_LAUNCH_CHECK("attn_decode_kernel");
     return LLM_OK;
+}
+
+template <bool FUSED>
+static int dispatch_decode(AdArgs a, int n_heads, int head_dim, void *ws, hipStream_t s) {
+    const int G = n_heads / a.n_kv_heads;
+#define AD_CASE(HD_, G_) \
+    if (head_dim == HD_ && G == G_) return launch_decode<HD_, G_, FUSED>(a, ws, s);
+    AD_CASE(128, 4)
+    AD_CASE(128, 8)
+    AD_CASE(128, 1)
+    AD_CASE(64, 4)
+    AD_CASE(64, 1)
+    AD_CASE(32, 4)
+    AD_CASE(32, 1)
+#undef AD_CASE
+    llm_set_error("llm_attn_decode: head_dim=%d with group size %d is not built", head_dim, G);
+    return LLM_ERR_INVALID;
 }
 
 extern "C" {
@@ -206,23 +357,38 @@ int llm_attn_decode(const uint16_t *q, const uint16_t *kc, const uint16_t *vc, u
     LLM_REQUIRE(max_pos > 0 && max_pos % 64 == 0, "llm_attn_decode: max_pos=%d must be a multiple of 64", max_pos);
     LLM_REQUIRE(ctx_dev || (ctx_host >= 1 && ctx_host <= max_pos), "llm_attn_decode: ctx=%d of %d", ctx_host, max_pos);
     LLM_REQUIRE(aligned16(q) && aligned16(kc) && aligned16(vc), "llm_attn_decode: pointers must be 16-byte aligned");
-    const int G = n_heads / n_kv_heads;
-    hipStream_t s = (hipStream_t)stream;
-    const half_t *qp = (const half_t *)q, *kp = (const half_t *)kc, *vp = (const half_t *)vc;
-    half_t *op = (half_t *)out;
-#define AD_CASE(HD_, G_)                                                                                   \
-    if (head_dim == HD_ && G == G_)                                                                        \
-        return launch_decode<HD_, G_>(qp, kp, vp, op, ctx_host, ctx_dev, n_kv_heads, max_pos, workspace, s);
-    AD_CASE(128, 4)
-    AD_CASE(128, 8)
-    AD_CASE(128, 1)
-    AD_CASE(64, 4)
-    AD_CASE(64, 1)
-    AD_CASE(32, 4)
-    AD_CASE(32, 1)
-#undef AD_CASE
-    llm_set_error("llm_attn_decode: head_dim=%d with group size %d is not built", head_dim, G);
-    return LLM_ERR_INVALID;
+    AdArgs a = {};
+    a.q = (const half_t *)q;
+    a.kc = (half_t *)kc;
+    a.vc = (half_t *)vc;
+    a.out = (half_t *)out;
+    a.pos_host = ctx_host - 1;
+    a.pos_dev = ctx_dev;
+    a.n_kv_heads = n_kv_heads;
+    a.max_pos = max_pos;
+    return dispatch_decode<false>(a, n_heads, head_dim, workspace, (hipStream_t)stream);
+}
+
+int llm_attn_decode_rope(const uint16_t *qkv, uint16_t *kc, uint16_t *vc, uint16_t *out, int pos_host,
+                         const int32_t *pos_dev, const float *table, int n_heads, int n_kv_heads, int head_dim,
+                         int max_pos, void *workspace, llm_stream_t stream) {
+    LLM_REQUIRE(qkv && kc && vc && out && table && workspace, "llm_attn_decode_rope: null pointer");
+    LLM_REQUIRE(n_kv_heads > 0 && n_heads % n_kv_heads == 0, "llm_attn_decode_rope: heads %d/%d", n_heads, n_kv_heads);
+    LLM_REQUIRE(max_pos > 0 && max_pos % 64 == 0, "llm_attn_decode_rope: max_pos=%d must be a multiple of 64", max_pos);
+    LLM_REQUIRE(pos_dev || (pos_host >= 0 && pos_host < max_pos), "llm_attn_decode_rope: position %d of %d", pos_host,
+                max_pos);
+    LLM_REQUIRE(aligned16(qkv) && aligned16(kc) && aligned16(vc), "llm_attn_decode_rope: pointers must be 16-byte aligned");
+    AdArgs a = {};
+    a.q = (const half_t *)qkv;
+    a.kc = (half_t *)kc;
+    a.vc = (half_t *)vc;
+    a.out = (half_t *)out;
+    a.table = table;
+    a.pos_host = pos_host;
+    a.pos_dev = pos_dev;
+    a.n_kv_heads = n_kv_heads;
+    a.max_pos = max_pos;
+    return dispatch_decode<true>(a, n_heads, head_dim, workspace, (hipStream_t)stream);
 }
 
 } // extern "C"

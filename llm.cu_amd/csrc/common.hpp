@@ -49,15 +49,42 @@ void llm_set_error(const char *fmt, ...) __attribute__((format(printf, 1, 2)));
 static inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 // ---- device helpers ---------------------------------------------------------
+// Cross-lane moves inside a row of 16 lanes run on the VALU's DPP path (no trip
+// through the LDS crossbar that __shfl uses).  Controls: quad_perm(1,0,3,2),
+// quad_perm(2,3,0,1), row_half_mirror, row_mirror.
+template <int CTRL> __device__ __forceinline__ float dpp_move(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
+
+// Sum over aligned groups of N lanes (N = 2, 4, 8 or 16); every lane of the group gets it.
+template <int N> __device__ __forceinline__ float group_sum(float v) {
+    static_assert(N == 1 || N == 2 || N == 4 || N == 8 || N == 16, "group size");
+    if (N >= 2) v += dpp_move<0xB1>(v);
+    if (N >= 4) v += dpp_move<0x4E>(v);
+    if (N >= 8) v += dpp_move<0x141>(v);
+    if (N >= 16) v += dpp_move<0x140>(v);
+    return v;
+}
+
+template <int N> __device__ __forceinline__ float group_max(float v) {
+    if (N >= 2) v = fmaxf(v, dpp_move<0xB1>(v));
+    if (N >= 4) v = fmaxf(v, dpp_move<0x4E>(v));
+    if (N >= 8) v = fmaxf(v, dpp_move<0x141>(v));
+    if (N >= 16) v = fmaxf(v, dpp_move<0x140>(v));
+    return v;
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off);
+    v = group_sum<16>(v);
+    v += __shfl_xor(v, 16);
+    v += __shfl_xor(v, 32);
     return v;
 }
 
 __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) v = fmaxf(v, __shfl_xor(v, off));
+    v = group_max<16>(v);
+    v = fmaxf(v, __shfl_xor(v, 16));
+    v = fmaxf(v, __shfl_xor(v, 32));
     return v;
 }
 

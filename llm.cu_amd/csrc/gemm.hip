@@ -17,9 +17,10 @@
 
 #include "common.hpp"
 
-int gemv_launch(const half_t *x, const half_t *w, const half_t *res, half_t *out, int N, int K, hipStream_t s);
-int gemv_swiglu_launch(const half_t *x, const half_t *wg, const half_t *wu, half_t *out, int N, int K,
-                       hipStream_t s);
+int gemv_launch(const half_t *x, const half_t *gain, double eps, const half_t *w, const half_t *res, half_t *out,
+                int N, int K, hipStream_t s);
+int gemv_swiglu_launch(const half_t *x, const half_t *gain, double eps, const half_t *wg, const half_t *wu,
+                       half_t *out, int N, int K, hipStream_t s);
 
 __device__ __forceinline__ float silu_g(float g) { return g / (1.0f + expf(-g)); }
 
@@ -286,7 +287,7 @@ int llm_linear(const uint16_t *x, int ldx, const uint16_t *w, const uint16_t *re
     hipStream_t s = (hipStream_t)stream;
     const half_t *xp = (const half_t *)x, *wp = (const half_t *)w, *rp = (const half_t *)residual;
     half_t *op = (half_t *)out;
-    if (T == 1) return gemv_launch(xp, wp, rp, op, N, K, s);
+    if (T == 1) return gemv_launch(xp, nullptr, 0.0, wp, rp, op, N, K, s);
     if (T <= 16 && K % (SK_WAVES * 32) == 0) {
         skinny_kernel<false><<<dim3((N + 15) / 16), dim3(SK_WAVES * 64), 0, s>>>(xp, ldx, wp, nullptr, rp, ldr, op,
                                                                                ldo, T, N, K);
@@ -307,7 +308,7 @@ int llm_linear_swiglu(const uint16_t *x, int ldx, const uint16_t *wgate, const u
     hipStream_t s = (hipStream_t)stream;
     const half_t *xp = (const half_t *)x, *gp = (const half_t *)wgate, *up = (const half_t *)wup;
     half_t *op = (half_t *)out;
-    if (T == 1) return gemv_swiglu_launch(xp, gp, up, op, N, K, s);
+    if (T == 1) return gemv_swiglu_launch(xp, nullptr, 0.0, gp, up, op, N, K, s);
     if (T <= 16 && K % (SK_WAVES * 32) == 0) {
         skinny_kernel<true><<<dim3((N + 15) / 16), dim3(SK_WAVES * 64), 0, s>>>(xp, ldx, gp, up, nullptr, 0, op, ldo,
                                                                               T, N, K);
@@ -317,6 +318,25 @@ int llm_linear_swiglu(const uint16_t *x, int ldx, const uint16_t *wgate, const u
     if (T <= 64 || N < 256) return gemm_launch<64, 64, 2, 2, 2>(xp, ldx, gp, up, nullptr, 0, op, ldo, T, N, K, s);
     if (T <= 128) return gemm_launch<128, 64, 2, 2, 2>(xp, ldx, gp, up, nullptr, 0, op, ldo, T, N, K, s);
     return gemm_launch<256, 128, 2, 2, 2>(xp, ldx, gp, up, nullptr, 0, op, ldo, T, N, K, s);
+}
+
+int llm_norm_linear(const uint16_t *x, const uint16_t *gain, double eps, const uint16_t *w, uint16_t *out, int N, int K,
+                    llm_stream_t stream) {
+    LLM_REQUIRE(x && gain && w && out, "llm_norm_linear: null pointer");
+    LLM_REQUIRE(N > 0 && K > 0, "llm_norm_linear: N=%d K=%d", N, K);
+    LLM_REQUIRE(aligned16(x) && aligned16(gain) && aligned16(w), "llm_norm_linear: pointers must be 16-byte aligned");
+    return gemv_launch((const half_t *)x, (const half_t *)gain, eps, (const half_t *)w, nullptr, (half_t *)out, N, K,
+                       (hipStream_t)stream);
+}
+
+int llm_norm_linear_swiglu(const uint16_t *x, const uint16_t *gain, double eps, const uint16_t *wgate,
+                           const uint16_t *wup, uint16_t *out, int N, int K, llm_stream_t stream) {
+    LLM_REQUIRE(x && gain && wgate && wup && out, "llm_norm_linear_swiglu: null pointer");
+    LLM_REQUIRE(N > 0 && K > 0, "llm_norm_linear_swiglu: N=%d K=%d", N, K);
+    LLM_REQUIRE(aligned16(x) && aligned16(gain) && aligned16(wgate) && aligned16(wup),
+                "llm_norm_linear_swiglu: pointers must be 16-byte aligned");
+    return gemv_swiglu_launch((const half_t *)x, (const half_t *)gain, eps, (const half_t *)wgate,
+                              (const half_t *)wup, (half_t *)out, N, K, (hipStream_t)stream);
 }
 
 } // extern "C"

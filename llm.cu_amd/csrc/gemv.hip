@@ -1,155 +1,178 @@
 // Bandwidth-bound projections for one token (decode): fp16 GEMV with 16-byte
-// coalesced weight loads, fp32 accumulation on v_dot2_f32_f16, wavefront
-// reductions; plus the fused SwiGLU pair and the LM head with greedy argmax.
+// coalesced, non-temporal weight loads, fp32 accumulation on v_dot2_f32_f16 and
+// wavefront reductions.  One kernel covers the plain projection (+ residual),
+// the fused SwiGLU pair and the LM head with greedy-argmax candidates, and each
+// can take the RMSNorm of its input on the way in.
 //
-// Layout: w is [N, K] row-major (the reference's [out, in]).  One wavefront
-// owns R consecutive rows at a time; lane l streams 16-byte pieces
-// k = 8l + 512j of each row, so a wavefront reads whole contiguous 1 KiB
-// spans of a row per load.  The activation vector sits in LDS.
+// Layout: w is [N, K] row-major (the reference's [out, in]).  A workgroup of 4
+// wavefronts handles 4*rpw rows, four adjacent rows at a time.  Lane l reads
+// the 16-byte pieces k = 8l + 512j of a row: every load instruction of a
+// wavefront covers a contiguous 1 KiB.  The activation vector (normalised if a
+// gain is given) sits in LDS; the first weight loads are issued before it is
+// staged so HBM is busy from the first cycle, and loads for the next span are
+// in flight while the current one is consumed.
 #include <cmath>
 
 #include "common.hpp"
+#include "rms_device.hpp"
 
 #define GEMV_THREADS 256
 #define GEMV_WAVES 4
+#define GEMV_U 4
+#define GEMV_SPAN (512 * GEMV_U)
+#define GEMV_NORM_R 4 // fused RMSNorm: K <= 4 * 4 * GEMV_THREADS = 4096
 
-__device__ __forceinline__ void stage_x(const half_t *__restrict__ x, half_t *xs, int K) {
-    for (int c = threadIdx.x * 8; c < K; c += GEMV_THREADS * 8) store8(xs + c, load8(x + c));
-    __syncthreads();
-}
+enum { GV_PLAIN = 0, GV_SWIGLU = 1, GV_LMHEAD = 2 };
 
-// Accumulates R rows against xs; U independent 16-byte loads per row in flight.
-template <int R, int U>
-__device__ __forceinline__ void gemv_rows(const half_t *const (&wp)[R], const half_t *xs, int K, int lane,
-                                          float (&acc)[R]) {
-    const int span = 512 * U;
-    const int kmain = K / span * span;
-    for (int k0 = 0; k0 < kmain; k0 += span) {
-        half8_t wv[R][U];
-#pragma unroll
-        for (int r = 0; r < R; ++r)
-#pragma unroll
-            for (int u = 0; u < U; ++u) wv[r][u] = load8(wp[r] + k0 + u * 512 + lane * 8);
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-            half8_t xv = load8(xs + k0 + u * 512 + lane * 8);
-#pragma unroll
-            for (int r = 0; r < R; ++r) acc[r] = dot8(wv[r][u], xv, acc[r]);
-        }
-    }
-    for (int k = kmain + lane * 8; k < K; k += 512) {
-        half8_t xv = load8(xs + k);
-#pragma unroll
-        for (int r = 0; r < R; ++r) acc[r] = dot8(load8(wp[r] + k), xv, acc[r]);
-    }
-}
+struct GemvArgs {
+    const half_t *x;     // [K]
+    const half_t *gain;  // [K] or null: RMSNorm fused into the staging of x
+    double eps;
+    const half_t *w;     // [N, K]
+    const half_t *w2;    // GV_SWIGLU: the up matrix (w is the gate)
+    const half_t *res;   // GV_PLAIN: optional residual [N]
+    half_t *out;         // [N] (GV_LMHEAD: the fp16 logits)
+    unsigned long long *cand; // GV_LMHEAD: one argmax candidate per workgroup
+    int N, K, rpw;
+};
 
-template <int R, int U>
-__global__ __launch_bounds__(GEMV_THREADS) void gemv_kernel(const half_t *__restrict__ x,
-                                                            const half_t *__restrict__ w,
-                                                            const half_t *__restrict__ res,
-                                                            half_t *__restrict__ out, int N, int K) {
-    extern __shared__ half_t xs[];
-    stage_x(x, xs, K);
-    const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
-    const int row0 = (blockIdx.x * GEMV_WAVES + wave) * R;
-    if (row0 >= N) return;
-    const half_t *wp[R];
-    float acc[R];
-#pragma unroll
-    for (int r = 0; r < R; ++r) {
-        int row = row0 + r < N ? row0 + r : N - 1;
-        wp[r] = w + (size_t)row * K;
-        acc[r] = 0.f;
-    }
-    gemv_rows<R, U>(wp, xs, K, lane, acc);
-#pragma unroll
-    for (int r = 0; r < R; ++r) {
-        float s = wave_sum(acc[r]);
-        if (lane == 0 && row0 + r < N) out[row0 + r] = finish(s, res ? res + row0 + r : nullptr);
-    }
+__device__ __forceinline__ half8_t load8_nt(const half_t *p) {
+    uint4_t v = __builtin_nontemporal_load(reinterpret_cast<const uint4_t *>(p));
+    return __builtin_bit_cast(half8_t, v);
 }
 
 __device__ __forceinline__ float silu_f(float g) { return g / (1.0f + expf(-g)); }
 
-template <int R, int U>
-__global__ __launch_bounds__(GEMV_THREADS) void gemv_swiglu_kernel(const half_t *__restrict__ x,
-                                                                   const half_t *__restrict__ wg,
-                                                                   const half_t *__restrict__ wu,
-                                                                   half_t *__restrict__ out, int N, int K) {
-    extern __shared__ half_t xs[];
-    stage_x(x, xs, K);
-    const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
-    const int row0 = (blockIdx.x * GEMV_WAVES + wave) * R;
-    if (row0 >= N) return;
-    const half_t *wp[2 * R];
-    float acc[2 * R];
-#pragma unroll
-    for (int r = 0; r < R; ++r) {
-        int row = row0 + r < N ? row0 + r : N - 1;
-        wp[r] = wg + (size_t)row * K;
-        wp[R + r] = wu + (size_t)row * K;
-        acc[r] = acc[R + r] = 0.f;
-    }
-    gemv_rows<2 * R, U>(wp, xs, K, lane, acc);
-#pragma unroll
-    for (int r = 0; r < R; ++r) {
-        float g = wave_sum(acc[r]);
-        float u = wave_sum(acc[R + r]);
-        if (lane == 0 && row0 + r < N) out[row0 + r] = (half_t)(silu_f(g) * u);
-    }
-}
-
-// LM head: logits for R rows per wavefront plus a per-block argmax candidate.
-// Candidates are packed (order key + 1) << 32 | ~index so that an unsigned
-// max picks the largest logit and, among equals, the lowest index; NaN packs
-// to 0 and never wins.
+// Candidates are packed (order key + 1) << 32 | ~index so that an unsigned max
+// picks the largest logit and, among equals, the lowest index; NaN packs to 0
+// and never wins.
 __device__ __forceinline__ unsigned long long pack_candidate(half_t h, int idx) {
     uint16_t bits = __builtin_bit_cast(uint16_t, h);
     if ((bits & 0x7fffu) > 0x7c00u) return 0ull;
     return ((unsigned long long)(f16_order_key(bits) + 1u) << 32) | (unsigned long long)(0xffffffffu - (uint32_t)idx);
 }
 
-template <int R, int U>
-__global__ __launch_bounds__(GEMV_THREADS) void lmhead_kernel(const half_t *__restrict__ x,
-                                                              const half_t *__restrict__ w,
-                                                              half_t *__restrict__ logits,
-                                                              unsigned long long *__restrict__ cand, int N,
-                                                              int K) {
-    extern __shared__ half_t xs[];
+template <int MODE>
+__global__ __launch_bounds__(GEMV_THREADS) void gemv_kernel(const GemvArgs a) {
+    constexpr int NW = MODE == GV_SWIGLU ? 2 : 1; // weight streams per row
+    extern __shared__ __attribute__((aligned(16))) half_t xs[];
+    __shared__ float red[GEMV_THREADS + 1];
     __shared__ unsigned long long best[GEMV_WAVES];
-    stage_x(x, xs, K);
+    const int K = a.K, N = a.N;
     const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
-    const int row0 = (blockIdx.x * GEMV_WAVES + wave) * R;
-    unsigned long long mine = 0ull;
-    if (row0 < N) {
-        const half_t *wp[R];
-        float acc[R];
+    // Row i of wavefront v in workgroup b is i*(4*grid) + 4*b + v: at any moment the
+    // whole grid reads one compact, advancing window of the matrix (DRAM pages
+    // stay open) instead of one far-apart stream per workgroup.
+    const int row_base = blockIdx.x * GEMV_WAVES + wave;
+    const int row_step = gridDim.x * GEMV_WAVES;
+    const int spr = (K + GEMV_SPAN - 1) / GEMV_SPAN; // spans per row
+    const int steps = a.rpw * spr;
+
+    half8_t buf[2][NW][GEMV_U];
+    // loads of step s (row i = s / spr, span s % spr) into buf[which]
+    auto issue = [&](int which, int i, int sp) {
+        int row = row_base + row_step * i;
+        row = row < N ? row : N - 1;
+        const size_t off = (size_t)row * K + sp * GEMV_SPAN + lane * 8;
 #pragma unroll
-        for (int r = 0; r < R; ++r) {
-            int row = row0 + r < N ? row0 + r : N - 1;
-            wp[r] = w + (size_t)row * K;
-            acc[r] = 0.f;
+        for (int u = 0; u < GEMV_U; ++u) {
+            const bool ok = sp * GEMV_SPAN + u * 512 + lane * 8 < K;
+            buf[which][0][u] = ok ? load8_nt(a.w + off + u * 512) : half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+            if (NW == 2) buf[which][NW - 1][u] = ok ? load8_nt(a.w2 + off + u * 512) : half8_t{0, 0, 0, 0, 0, 0, 0, 0};
         }
-        gemv_rows<R, U>(wp, xs, K, lane, acc);
+    };
+
+    // cursors: (li, lsp) = next step to load, (i, sp) = step being consumed
+    int li = 0, lsp = 0, loaded = 0;
+    auto issue_next = [&](int which) {
+        if (loaded < steps) {
+            issue(which, li, lsp);
+            ++loaded;
+            if (++lsp == spr) { lsp = 0; ++li; }
+        }
+    };
+
+    // the activation loads go out first, then two steps of weights; only then
+    // does anything wait (the norm's reduction), so HBM is busy throughout
+    RmsRow<GEMV_NORM_R> xr;
+    half8_t xraw[4];
+    if (a.gain) {
+        rms_load<GEMV_THREADS, GEMV_NORM_R>(a.x, a.gain, K, xr);
+    } else {
 #pragma unroll
-        for (int r = 0; r < R; ++r) {
-            float s = wave_sum(acc[r]);
-            if (row0 + r < N) {
-                half_t h = (half_t)s;
-                if (lane == 0) logits[row0 + r] = h;
-                unsigned long long c = pack_candidate(h, row0 + r);
-                mine = c > mine ? c : mine;
-            }
+        for (int j = 0; j < 4; ++j) {
+            const int c = (threadIdx.x + GEMV_THREADS * j) * 8;
+            if (c < K) xraw[j] = load8(a.x + c);
         }
     }
-    if (lane == 0) best[wave] = mine;
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        unsigned long long b = best[0];
+    issue_next(0);
+    issue_next(1);
+    if (a.gain) {
+        rms_finish<GEMV_THREADS, GEMV_NORM_R>(xr, xs, K, a.eps, red);
+    } else {
 #pragma unroll
-        for (int i = 1; i < GEMV_WAVES; ++i) b = best[i] > b ? best[i] : b;
-        cand[blockIdx.x] = b;
+        for (int j = 0; j < 4; ++j) {
+            const int c = (threadIdx.x + GEMV_THREADS * j) * 8;
+            if (c < K) store8(xs + c, xraw[j]);
+        }
+        for (int c = (threadIdx.x + GEMV_THREADS * 4) * 8; c < K; c += GEMV_THREADS * 8) store8(xs + c, load8(a.x + c));
+    }
+    __syncthreads();
+
+    float acc[NW];
+#pragma unroll
+    for (int j = 0; j < NW; ++j) acc[j] = 0.f;
+    unsigned long long mine = 0ull;
+    int i = 0, sp = 0;
+    auto consume = [&](int which) {
+#pragma unroll
+        for (int u = 0; u < GEMV_U; ++u) {
+            const int k = sp * GEMV_SPAN + u * 512 + lane * 8;
+            if (k < K) {
+                const half8_t xv = load8(xs + k);
+#pragma unroll
+                for (int j = 0; j < NW; ++j) acc[j] = dot8(buf[which][j][u], xv, acc[j]);
+            }
+        }
+        if (sp == spr - 1) { // row finished
+            const int row = row_base + row_step * i;
+            float s0 = wave_sum(acc[0]);
+            float s1 = NW == 2 ? wave_sum(acc[NW - 1]) : 0.f;
+            if (row < N) {
+                if (MODE == GV_SWIGLU) {
+                    if (lane == 0) a.out[row] = (half_t)(silu_f(s0) * s1);
+                } else if (MODE == GV_LMHEAD) {
+                    const half_t h = (half_t)s0;
+                    if (lane == 0) a.out[row] = h;
+                    const unsigned long long c = pack_candidate(h, row);
+                    mine = c > mine ? c : mine;
+                } else {
+                    if (lane == 0) a.out[row] = finish(s0, a.res ? a.res + row : nullptr);
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < NW; ++j) acc[j] = 0.f;
+        }
+        if (++sp == spr) { sp = 0; ++i; }
+    };
+    // two steps per trip: each register buffer is refilled right after it is consumed
+    for (int s = 0; s < steps; s += 2) {
+        consume(0);
+        issue_next(0);
+        if (s + 1 < steps) {
+            consume(1);
+            issue_next(1);
+        }
+    }
+    if (MODE == GV_LMHEAD) {
+        if (lane == 0) best[wave] = mine;
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            unsigned long long b = best[0];
+#pragma unroll
+            for (int v = 1; v < GEMV_WAVES; ++v) b = best[v] > b ? best[v] : b;
+            a.cand[blockIdx.x] = b;
+        }
     }
 }
 
@@ -198,54 +221,70 @@ __global__ __launch_bounds__(1024) void argmax_final_kernel(const unsigned long 
 }
 
 // ---------------------------------------------------------------------------
-int gemv_launch(const half_t *x, const half_t *w, const half_t *res, half_t *out, int N, int K, hipStream_t s) {
-    const size_t smem = (size_t)K * sizeof(half_t);
-    LLM_REQUIRE(smem <= 64 * 1024, "GEMV: K=%d does not fit the 64 KiB LDS staging", K);
-    constexpr int R = 2, U = 4;
-    const int blocks = (N + GEMV_WAVES * R - 1) / (GEMV_WAVES * R);
-    gemv_kernel<R, U><<<dim3(blocks), dim3(GEMV_THREADS), smem, s>>>(x, w, res, out, N, K);
+// Rows per wavefront, from sweeps on MI355X at the LLaMA3-8B shapes: many small
+// workgroups win (the hardware keeps refilling CUs as wavefronts retire); only
+// the norm-fused QKV projection and the 128K-row LM head amortise their
+// per-workgroup prologue over more than one row.
+static int rows_per_wave(int mode, int N, bool norm) {
+    if (mode == GV_LMHEAD) return N >= 32768 ? 3 : 1;
+    if (mode == GV_PLAIN && norm && N >= 6144) return 2;
+    return 1;
+}
+
+static int gemv_blocks(int N, int rpw) { return (N + GEMV_WAVES * rpw - 1) / (GEMV_WAVES * rpw); }
+
+template <int MODE> static int gemv_dispatch(GemvArgs a, hipStream_t s) {
+    const size_t smem = (size_t)a.K * sizeof(half_t);
+    LLM_REQUIRE(a.K % 8 == 0 && smem <= 56 * 1024, "GEMV: K=%d must be a multiple of 8 and fit 56 KiB of LDS", a.K);
+    LLM_REQUIRE(!a.gain || (rms_shape_ok(a.K) && a.K <= 4 * GEMV_NORM_R * GEMV_THREADS),
+                "GEMV with RMSNorm: K=%d (need K/4 a power of two in [64, %d])", a.K, GEMV_NORM_R * GEMV_THREADS);
+    gemv_kernel<MODE><<<dim3(gemv_blocks(a.N, a.rpw)), dim3(GEMV_THREADS), smem, s>>>(a);
     LLM_LAUNCH_CHECK("gemv_kernel");
     return LLM_OK;
 }
 
-int gemv_swiglu_launch(const half_t *x, const half_t *wg, const half_t *wu, half_t *out, int N, int K,
-                       hipStream_t s) {
-    const size_t smem = (size_t)K * sizeof(half_t);
-    LLM_REQUIRE(smem <= 64 * 1024, "GEMV: K=%d does not fit the 64 KiB LDS staging", K);
-    constexpr int R = 1, U = 4;
-    const int blocks = (N + GEMV_WAVES * R - 1) / (GEMV_WAVES * R);
-    gemv_swiglu_kernel<R, U><<<dim3(blocks), dim3(GEMV_THREADS), smem, s>>>(x, wg, wu, out, N, K);
-    LLM_LAUNCH_CHECK("gemv_swiglu_kernel");
-    return LLM_OK;
+int gemv_launch(const half_t *x, const half_t *gain, double eps, const half_t *w, const half_t *res, half_t *out,
+                int N, int K, hipStream_t s) {
+    GemvArgs a = {x, gain, eps, w, nullptr, res, out, nullptr, N, K, rows_per_wave(GV_PLAIN, N, gain != nullptr)};
+    return gemv_dispatch<GV_PLAIN>(a, s);
+}
+
+int gemv_swiglu_launch(const half_t *x, const half_t *gain, double eps, const half_t *wg, const half_t *wu,
+                       half_t *out, int N, int K, hipStream_t s) {
+    GemvArgs a = {x, gain, eps, wg, wu, nullptr, out, nullptr, N, K, rows_per_wave(GV_SWIGLU, N, gain != nullptr)};
+    return gemv_dispatch<GV_SWIGLU>(a, s);
 }
 
 extern "C" {
 
 size_t llm_lmhead_workspace_bytes(int vocab) {
-    constexpr int R = 2;
-    size_t blocks = ((size_t)vocab + GEMV_WAVES * R - 1) / (GEMV_WAVES * R);
+    size_t blocks = (size_t)gemv_blocks(vocab, 1); // upper bound for any rows-per-wave choice
     if (blocks < 1024) blocks = 1024;
     return blocks * sizeof(unsigned long long);
 }
 
-int llm_lmhead_argmax(const uint16_t *x, const uint16_t *w, uint16_t *logits, int32_t *token, int32_t *tokens,
-                      int32_t *pos, int vocab, int K, void *workspace, llm_stream_t stream) {
+int llm_norm_lmhead_argmax(const uint16_t *x, const uint16_t *gain, double eps, const uint16_t *w, uint16_t *logits,
+                           int32_t *token, int32_t *tokens, int32_t *pos, int vocab, int K, void *workspace,
+                           llm_stream_t stream) {
     LLM_REQUIRE(x && w && logits && token && workspace, "llm_lmhead_argmax: null pointer");
-    LLM_REQUIRE(vocab > 0 && K > 0 && K % 8 == 0, "llm_lmhead_argmax: vocab=%d K=%d", vocab, K);
-    LLM_REQUIRE(aligned16(x) && aligned16(w), "llm_lmhead_argmax: pointers must be 16-byte aligned");
+    LLM_REQUIRE(vocab > 0 && K > 0, "llm_lmhead_argmax: vocab=%d K=%d", vocab, K);
+    LLM_REQUIRE(aligned16(x) && aligned16(w) && (!gain || aligned16(gain)), "llm_lmhead_argmax: pointers must be 16-byte aligned");
     LLM_REQUIRE((tokens == nullptr) == (pos == nullptr), "llm_lmhead_argmax: tokens and pos go together");
-    const size_t smem = (size_t)K * sizeof(half_t);
-    LLM_REQUIRE(smem <= 64 * 1024, "llm_lmhead_argmax: K=%d does not fit the LDS staging", K);
-    constexpr int R = 2, U = 4;
-    const int blocks = (vocab + GEMV_WAVES * R - 1) / (GEMV_WAVES * R);
     hipStream_t s = (hipStream_t)stream;
-    lmhead_kernel<R, U><<<dim3(blocks), dim3(GEMV_THREADS), smem, s>>>(
-        (const half_t *)x, (const half_t *)w, (half_t *)logits, (unsigned long long *)workspace, vocab, K);
-    LLM_LAUNCH_CHECK("lmhead_kernel");
-    argmax_final_kernel<<<dim3(1), dim3(1024), 0, s>>>((const unsigned long long *)workspace, blocks, token, tokens,
-                                                       pos);
+    const int rpw = rows_per_wave(GV_LMHEAD, vocab, gain != nullptr);
+    GemvArgs a = {(const half_t *)x, (const half_t *)gain, eps, (const half_t *)w, nullptr, nullptr, (half_t *)logits,
+                  (unsigned long long *)workspace, vocab, K, rpw};
+    int rc = gemv_dispatch<GV_LMHEAD>(a, s);
+    if (rc != LLM_OK) return rc;
+    argmax_final_kernel<<<dim3(1), dim3(1024), 0, s>>>((const unsigned long long *)workspace, gemv_blocks(vocab, rpw),
+                                                       token, tokens, pos);
     LLM_LAUNCH_CHECK("argmax_final_kernel");
     return LLM_OK;
+}
+
+int llm_lmhead_argmax(const uint16_t *x, const uint16_t *w, uint16_t *logits, int32_t *token, int32_t *tokens,
+                      int32_t *pos, int vocab, int K, void *workspace, llm_stream_t stream) {
+    return llm_norm_lmhead_argmax(x, nullptr, 0.0, w, logits, token, tokens, pos, vocab, K, workspace, stream);
 }
 
 int llm_argmax_f16(const uint16_t *logits, int n, int32_t *token, void *workspace, llm_stream_t stream) {

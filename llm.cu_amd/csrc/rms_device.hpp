@@ -21,21 +21,45 @@ static inline bool rms_shape_ok(int d) {
 
 #define RMS_MAX_R 16 // slots per thread: d/4/THREADS <= 16  (d <= 16384 at 256 threads)
 
-// Returns ss for the row; every thread gets the value.  `vals` receives the
-// thread's 4*R input elements (slot j at vals[4j..4j+3]).
-template <int THREADS>
-__device__ __forceinline__ float rms_sum_squares(const half_t *__restrict__ xrow, int d, float *red,
-                                                 half4_t *vals, int &R_out) {
+// A thread's share of one row: slot j covers elements 4*(t + THREADS*j)..+3.
+template <int MAXR = RMS_MAX_R> struct RmsRow {
+    half4_t x[MAXR];
+    half4_t g[MAXR];
+    int R; // live slots of this thread (0 for spare threads of a narrow row)
+};
+
+// Issues the loads of the row (and of the gains when given) and returns at
+// once, so the caller can put other loads in flight before rms_finish waits.
+template <int THREADS, int MAXR>
+__device__ __forceinline__ void rms_load(const half_t *__restrict__ xrow, const half_t *__restrict__ gain, int d,
+                                         RmsRow<MAXR> &r) {
     const int t = threadIdx.x;
     const int n = d / 4;
-    const int R = n / THREADS; // power of two >= 1
-    R_out = R;
-    float p[RMS_MAX_R];
+    // fewer slots than threads: the spare threads hold zero slots, which the
+    // stride-halving tree folds in without changing any partial sum
+    const int R = n >= THREADS ? n / THREADS : 1; // power of two >= 1
+    r.R = t < n ? R : 0;
 #pragma unroll
-    for (int j = 0; j < RMS_MAX_R; ++j) {
-        if (j < R) {
-            half4_t v = *reinterpret_cast<const half4_t *>(xrow + 4 * (size_t)(t + THREADS * j));
-            vals[j] = v;
+    for (int j = 0; j < MAXR; ++j) {
+        if (j < r.R) {
+            const size_t e = 4 * (size_t)(t + THREADS * j);
+            r.x[j] = *reinterpret_cast<const half4_t *>(xrow + e);
+            if (gain) r.g[j] = *reinterpret_cast<const half4_t *>(gain + e);
+        }
+    }
+}
+
+// Sum of squares of the loaded row in the reference's order; every thread gets it.
+template <int THREADS, int MAXR>
+__device__ __forceinline__ float rms_sum_squares(const RmsRow<MAXR> &r, int d, float *red) {
+    const int t = threadIdx.x;
+    const int n = d / 4;
+    const int R = n >= THREADS ? n / THREADS : 1;
+    float p[MAXR];
+#pragma unroll
+    for (int j = 0; j < MAXR; ++j) {
+        if (j < r.R) {
+            const half4_t v = r.x[j];
             float a = (float)v[0], b = (float)v[1], c = (float)v[2], e = (float)v[3];
             p[j] = ((a * a + b * b) + c * c) + e * e;
         } else {
@@ -44,10 +68,10 @@ __device__ __forceinline__ float rms_sum_squares(const half_t *__restrict__ xrow
     }
     // top index bits live in j
 #pragma unroll
-    for (int off = RMS_MAX_R / 2; off >= 1; off >>= 1) {
+    for (int off = MAXR / 2; off >= 1; off >>= 1) {
         if (off < R) {
 #pragma unroll
-            for (int j = 0; j < RMS_MAX_R / 2; ++j)
+            for (int j = 0; j < (MAXR > 1 ? MAXR / 2 : 1); ++j)
                 if (j < off) p[j] += p[j + off];
         }
     }
@@ -83,24 +107,28 @@ __device__ __forceinline__ float rms_from_ss(float ss, int d, double eps) {
 
 // y = fp16((x * g) / rms): multiply, then a correctly rounded divide
 // (inference.cu:355-358).  dst may be global or LDS memory.
+template <int THREADS, int MAXR>
+__device__ __forceinline__ void rms_finish(const RmsRow<MAXR> &r, half_t *dst, int d, double eps, float *red) {
+    const float ss = rms_sum_squares<THREADS, MAXR>(r, d, red);
+    const float rms = rms_from_ss(ss, d, eps);
+    const int t = threadIdx.x;
+#pragma unroll
+    for (int j = 0; j < MAXR; ++j) {
+        if (j < r.R) {
+            const size_t e = 4 * (size_t)(t + THREADS * j);
+            half4_t o;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) o[k] = (half_t)(((float)r.x[j][k] * (float)r.g[j][k]) / rms);
+            *reinterpret_cast<half4_t *>(dst + e) = o;
+        }
+    }
+}
+
 template <int THREADS>
 __device__ __forceinline__ void rms_normalise_row(const half_t *__restrict__ xrow,
                                                   const half_t *__restrict__ gain, half_t *dst, int d,
                                                   double eps, float *red) {
-    half4_t vals[RMS_MAX_R];
-    int R;
-    float ss = rms_sum_squares<THREADS>(xrow, d, red, vals, R);
-    float rms = rms_from_ss(ss, d, eps);
-    const int t = threadIdx.x;
-#pragma unroll
-    for (int j = 0; j < RMS_MAX_R; ++j) {
-        if (j < R) {
-            const size_t e = 4 * (size_t)(t + THREADS * j);
-            half4_t g = *reinterpret_cast<const half4_t *>(gain + e);
-            half4_t o;
-#pragma unroll
-            for (int k = 0; k < 4; ++k) o[k] = (half_t)(((float)vals[j][k] * (float)g[k]) / rms);
-            *reinterpret_cast<half4_t *>(dst + e) = o;
-        }
-    }
+    RmsRow<RMS_MAX_R> r;
+    rms_load<THREADS, RMS_MAX_R>(xrow, gain, d, r);
+    rms_finish<THREADS, RMS_MAX_R>(r, dst, d, eps, red);
 }

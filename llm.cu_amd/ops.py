@@ -180,3 +180,47 @@ class Timer:
         ms = C.c_float(0)
         check(lib().llm_event_elapsed_ms(self.e0, self.e1, C.byref(ms)))
         return ms.value / iters
+
+
+def norm_linear(x, gain, w, eps=1e-5):
+    x, gain, w = _u16(x).reshape(-1), _u16(gain), _u16(w)
+    N, K = w.shape
+    d_x, d_g, d_w, d_o = DevBuf.from_host(x), DevBuf.from_host(gain), DevBuf.from_host(w), DevBuf((1, N), np.uint16)
+    check(lib().llm_norm_linear(d_x.ptr, d_g.ptr, eps, d_w.ptr, d_o.ptr, N, K, None))
+    return d_o.download()
+
+
+def norm_linear_swiglu(x, gain, wgate, wup, eps=1e-5):
+    x, gain, wgate, wup = _u16(x).reshape(-1), _u16(gain), _u16(wgate), _u16(wup)
+    N, K = wgate.shape
+    d_x, d_g = DevBuf.from_host(x), DevBuf.from_host(gain)
+    d_a, d_b, d_o = DevBuf.from_host(wgate), DevBuf.from_host(wup), DevBuf((1, N), np.uint16)
+    check(lib().llm_norm_linear_swiglu(d_x.ptr, d_g.ptr, eps, d_a.ptr, d_b.ptr, d_o.ptr, N, K, None))
+    return d_o.download()
+
+
+def norm_lmhead_argmax(x, gain, w, eps=1e-5):
+    x, gain, w = _u16(x).reshape(-1), _u16(gain), _u16(w)
+    vocab, K = w.shape
+    d_x, d_g, d_w = DevBuf.from_host(x), DevBuf.from_host(gain), DevBuf.from_host(w)
+    d_l, d_t = DevBuf((vocab,), np.uint16), DevBuf((1,), np.int32)
+    d_ws = DevBuf((lib().llm_lmhead_workspace_bytes(vocab),), np.uint8)
+    check(lib().llm_norm_lmhead_argmax(d_x.ptr, d_g.ptr, eps, d_w.ptr, d_l.ptr, d_t.ptr, None, None, vocab, K,
+                                       d_ws.ptr, None))
+    return int(d_t.download()[0]), d_l.download()
+
+
+def attn_decode_rope(qkv, kc, vc, pos, n_heads, n_kv_heads, head_dim, theta=500000.0, repeats=1):
+    """Returns (out [Hq*hd], K cache, V cache) after rope + append + attention at position pos."""
+    qkv, kc, vc = _u16(qkv).reshape(-1), _u16(kc), _u16(vc)
+    max_pos = kc.shape[1]
+    d_q, d_k, d_v = DevBuf.from_host(qkv), DevBuf.from_host(kc), DevBuf.from_host(vc)
+    d_o = DevBuf((n_heads * head_dim,), np.uint16)
+    d_t = DevBuf.from_host(rope_table(max_pos, head_dim, theta))
+    wsb = (lib().llm_attn_decode_workspace_bytes(n_heads, head_dim) + 3) // 4 * 4
+    d_ws = DevBuf((wsb // 4,), np.uint32)
+    d_ws.zero()
+    for _ in range(repeats):
+        check(lib().llm_attn_decode_rope(d_q.ptr, d_k.ptr, d_v.ptr, d_o.ptr, pos, None, d_t.ptr, n_heads, n_kv_heads,
+                                         head_dim, max_pos, d_ws.ptr, None))
+    return d_o.download(), d_k.download(), d_v.download()

@@ -6,7 +6,8 @@
 //
 // Layer graph (inference.cu:157-186), with the reference's extra passes folded
 // into neighbours where the result is the same bits:
-//   save residual + norm      -> llm_rmsnorm into a second buffer (x stays the residual)
+//   save residual + norm      -> llm_rmsnorm into a second buffer (x stays the residual);
+//                                for one row, folded into the next projection
 //   Q, K, V (3 launches)      -> one projection over the adjacent q|k|v weights
 //   RoPE(Q), RoPE(K)          -> llm_rope_kv_append (also writes the KV cache)
 //   scores, softmax, P.V      -> llm_attn_prefill / llm_attn_decode over the cache
@@ -110,40 +111,61 @@ void issue_pass(Engine *e, const Llama3 *m, int T, int pos0, bool dev_pos, bool 
 
     llama3_check(llm_embed_gather(m->embed_tokens->d_fp16_tensor, e->d_tokens + p0, pd, e->x, T, d, c.vocab, s),
                  "llm_embed_gather");
-    for (int l = 0; l < c.n_layers; ++l) {
-        const LayerW w = layer_w(m, l);
-        llm_half *kc = e->kc + (size_t)l * e->kv_layer_elems, *vc = e->vc + (size_t)l * e->kv_layer_elems;
-        llama3_check(llm_rmsnorm(e->x, w.in_ln, e->xn, T, d, c.rms_eps, s), "llm_rmsnorm");
-        if (w.wk == w.wq + (size_t)qd * d && w.wv == w.wk + (size_t)kvd * d) {
-            llama3_check(llm_linear(e->xn, d, w.wq, nullptr, 0, e->qkv, QKV, T, QKV, d, s), "llm_linear(qkv)");
-        } else {
-            llama3_check(llm_linear(e->xn, d, w.wq, nullptr, 0, e->qkv, QKV, T, qd, d, s), "llm_linear(q)");
-            llama3_check(llm_linear(e->xn, d, w.wk, nullptr, 0, e->qkv + qd, QKV, T, kvd, d, s), "llm_linear(k)");
-            llama3_check(llm_linear(e->xn, d, w.wv, nullptr, 0, e->qkv + qd + kvd, QKV, T, kvd, d, s), "llm_linear(v)");
+    const llm_half *final_gain = m->norm->d_fp16_tensor;
+    if (T == 1) {
+        // decode step: 5 launches per layer (norm folded into the projections, RoPE + cache append
+        // folded into the attention, residual adds in the projection epilogues)
+        for (int l = 0; l < c.n_layers; ++l) {
+            const LayerW w = layer_w(m, l);
+            llm_half *kc = e->kc + (size_t)l * e->kv_layer_elems, *vc = e->vc + (size_t)l * e->kv_layer_elems;
+            if (w.wk == w.wq + (size_t)qd * d && w.wv == w.wk + (size_t)kvd * d) {
+                llama3_check(llm_norm_linear(e->x, w.in_ln, c.rms_eps, w.wq, e->qkv, QKV, d, s), "llm_norm_linear(qkv)");
+            } else {
+                llama3_check(llm_norm_linear(e->x, w.in_ln, c.rms_eps, w.wq, e->qkv, qd, d, s), "llm_norm_linear(q)");
+                llama3_check(llm_norm_linear(e->x, w.in_ln, c.rms_eps, w.wk, e->qkv + qd, kvd, d, s), "llm_norm_linear(k)");
+                llama3_check(llm_norm_linear(e->x, w.in_ln, c.rms_eps, w.wv, e->qkv + qd + kvd, kvd, d, s),
+                             "llm_norm_linear(v)");
+            }
+            llama3_check(llm_attn_decode_rope(e->qkv, kc, vc, e->attn, p0, pd, e->rope_table, Hq, Hkv, hd, c.max_pos,
+                                              e->ws_attn, s),
+                         "llm_attn_decode_rope");
+            llama3_check(llm_linear(e->attn, qd, w.wo, e->x, d, e->x, d, 1, d, qd, s), "llm_linear(o)");
+            llama3_check(llm_norm_linear_swiglu(e->x, w.post_ln, c.rms_eps, w.wg, w.wu, e->ffn, F, d, s),
+                         "llm_norm_linear_swiglu");
+            llama3_check(llm_linear(e->ffn, F, w.wd, e->x, d, e->x, d, 1, d, F, s), "llm_linear(down)");
+            if (trace)
+                llama3_check(llm_memcpy_d2d(e->trace_dev + (size_t)l * d, e->x, sizeof(llm_half) * (size_t)d, s),
+                             "trace copy");
         }
-        llama3_check(llm_rope_kv_append(e->qkv, kc, vc, T, Hq, Hkv, hd, p0, pd, e->rope_table, c.max_pos, s),
-                     "llm_rope_kv_append");
-        if (T == 1) {
-            llama3_check(llm_attn_decode(e->qkv, kc, vc, e->attn, p0 + 1, pd, Hq, Hkv, hd, c.max_pos, e->ws_attn, s),
-                         "llm_attn_decode");
-        } else {
+    } else {
+        for (int l = 0; l < c.n_layers; ++l) {
+            const LayerW w = layer_w(m, l);
+            llm_half *kc = e->kc + (size_t)l * e->kv_layer_elems, *vc = e->vc + (size_t)l * e->kv_layer_elems;
+            llama3_check(llm_rmsnorm(e->x, w.in_ln, e->xn, T, d, c.rms_eps, s), "llm_rmsnorm");
+            if (w.wk == w.wq + (size_t)qd * d && w.wv == w.wk + (size_t)kvd * d) {
+                llama3_check(llm_linear(e->xn, d, w.wq, nullptr, 0, e->qkv, QKV, T, QKV, d, s), "llm_linear(qkv)");
+            } else {
+                llama3_check(llm_linear(e->xn, d, w.wq, nullptr, 0, e->qkv, QKV, T, qd, d, s), "llm_linear(q)");
+                llama3_check(llm_linear(e->xn, d, w.wk, nullptr, 0, e->qkv + qd, QKV, T, kvd, d, s), "llm_linear(k)");
+                llama3_check(llm_linear(e->xn, d, w.wv, nullptr, 0, e->qkv + qd + kvd, QKV, T, kvd, d, s), "llm_linear(v)");
+            }
+            llama3_check(llm_rope_kv_append(e->qkv, kc, vc, T, Hq, Hkv, hd, p0, pd, e->rope_table, c.max_pos, s),
+                         "llm_rope_kv_append");
             llama3_check(llm_attn_prefill(e->qkv, QKV, kc, vc, e->attn, qd, T, p0, Hq, Hkv, hd, c.max_pos, s),
                          "llm_attn_prefill");
+            llama3_check(llm_linear(e->attn, qd, w.wo, e->x, d, e->x, d, T, d, qd, s), "llm_linear(o)");
+            llama3_check(llm_rmsnorm(e->x, w.post_ln, e->xn, T, d, c.rms_eps, s), "llm_rmsnorm");
+            llama3_check(llm_linear_swiglu(e->xn, d, w.wg, w.wu, e->ffn, F, T, F, d, s), "llm_linear_swiglu");
+            llama3_check(llm_linear(e->ffn, F, w.wd, e->x, d, e->x, d, T, d, F, s), "llm_linear(down)");
+            if (trace)
+                llama3_check(llm_memcpy_d2d(e->trace_dev + (size_t)l * T * d, e->x, sizeof(llm_half) * (size_t)T * d, s),
+                             "trace copy");
         }
-        llama3_check(llm_linear(e->attn, qd, w.wo, e->x, d, e->x, d, T, d, qd, s), "llm_linear(o)");
-        llama3_check(llm_rmsnorm(e->x, w.post_ln, e->xn, T, d, c.rms_eps, s), "llm_rmsnorm");
-        llama3_check(llm_linear_swiglu(e->xn, d, w.wg, w.wu, e->ffn, F, T, F, d, s), "llm_linear_swiglu");
-        llama3_check(llm_linear(e->ffn, F, w.wd, e->x, d, e->x, d, T, d, F, s), "llm_linear(down)");
-        if (trace)
-            llama3_check(llm_memcpy_d2d(e->trace_dev + (size_t)l * T * d, e->x, sizeof(llm_half) * (size_t)T * d, s),
-                         "trace copy");
     }
-    // final norm on the last row only (the reference norms all rows and reads the last)
-    llama3_check(llm_rmsnorm(e->x + (size_t)(T - 1) * d, m->norm->d_fp16_tensor, e->xn, 1, d, c.rms_eps, s),
-                 "llm_rmsnorm(final)");
-    llama3_check(llm_lmhead_argmax(e->xn, m->lm_head->d_fp16_tensor, e->logits, e->d_token, e->d_tokens, e->d_pos,
-                                   c.vocab, d, e->ws_lm, s),
-                 "llm_lmhead_argmax");
+    // final norm on the last row only (the reference norms all rows and reads the last), folded into the LM head
+    llama3_check(llm_norm_lmhead_argmax(e->x + (size_t)(T - 1) * d, final_gain, c.rms_eps, m->lm_head->d_fp16_tensor,
+                                        e->logits, e->d_token, e->d_tokens, e->d_pos, c.vocab, d, e->ws_lm, s),
+                 "llm_norm_lmhead_argmax");
 }
 
 void drop_graph(Engine *e) {

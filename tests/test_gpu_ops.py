@@ -332,3 +332,67 @@ def test_attn_prefill_8192_last_rows_and_uniform_key_property(gpu):
     for h in (0, 5, 31):
         kv = h // 4
         assert np.allclose(out[:, h * hd:(h + 1) * hd], csum[:, kv * hd:(kv + 1) * hd], atol=5e-3)
+
+
+# ---- the decode step's fused entry points give the bits of the unfused sequence ------------------------------
+@pytest.mark.parametrize("K,N", [(4096, 6144), (256, 384)])
+def test_norm_linear_equals_rmsnorm_then_linear(gpu, K, N):
+    rng = np.random.default_rng(K)
+    x = H.bits(2.0 * rng.standard_normal((1, K)))
+    g = H.bits(1.0 + 0.1 * rng.standard_normal(K))
+    w = H.bits(0.02 * rng.standard_normal((N, K), dtype=np.float32))
+    got = gpu.ops.norm_linear(x, g, w)
+    assert np.array_equal(got, gpu.ops.linear(gpu.ops.rmsnorm(x, g), w))
+    assert H.mixed_err(got, orc.linear(orc.rmsnorm(x, g), w)) <= TIGHT
+
+
+@pytest.mark.parametrize("K,N", [(4096, 14336), (256, 768)])
+def test_norm_linear_swiglu_equals_unfused(gpu, K, N):
+    rng = np.random.default_rng(K + 1)
+    x = H.bits(2.0 * rng.standard_normal((1, K)))
+    g = H.bits(1.0 + 0.1 * rng.standard_normal(K))
+    wg = H.bits(0.02 * rng.standard_normal((N, K), dtype=np.float32))
+    wu = H.bits(0.02 * rng.standard_normal((N, K), dtype=np.float32))
+    got = gpu.ops.norm_linear_swiglu(x, g, wg, wu)
+    assert np.array_equal(got, gpu.ops.linear_swiglu(gpu.ops.rmsnorm(x, g), wg, wu))
+    assert H.mixed_err(got, orc.linear_swiglu(orc.rmsnorm(x, g), wg, wu)) <= TOL
+
+
+def test_norm_lmhead_argmax_equals_unfused(gpu):
+    K, V = 4096, 128256
+    rng = np.random.default_rng(13)
+    x = H.bits(3.0 * rng.standard_normal((1, K)))
+    g = H.bits(1.0 + 0.1 * rng.standard_normal(K))
+    w = H.bits(0.02 * rng.standard_normal((V, K), dtype=np.float32))
+    tok, logits = gpu.ops.norm_lmhead_argmax(x, g, w)
+    tok2, logits2 = gpu.ops.lmhead_argmax(gpu.ops.rmsnorm(x, g), w)
+    assert tok == tok2 == orc.argmax_f16(logits) and np.array_equal(logits, logits2)
+
+
+@pytest.mark.parametrize("pos,max_pos,Hq,Hkv,hd", [(0, 64, 8, 2, 32), (37, 64, 8, 2, 32), (0, 2048, 32, 8, 128),
+                                                   (300, 2048, 32, 8, 128), (511, 2048, 32, 8, 128),
+                                                   (512, 2048, 32, 8, 128), (1500, 2048, 32, 8, 128),
+                                                   (8447, 8704, 32, 8, 128)])
+def test_attn_decode_rope_fused(gpu, pos, max_pos, Hq, Hkv, hd):
+    """RoPE + cache append + attention in one launch == llm_rope_kv_append then llm_attn_decode, and == oracle."""
+    rng = np.random.default_rng(pos + hd)
+    qd, kvd = Hq * hd, Hkv * hd
+    # cache rows 0..pos-1 hold earlier (already rotated) keys and values
+    k_old = H.bits(rng.standard_normal((pos, kvd)))
+    v_old = H.bits(rng.standard_normal((pos, kvd)))
+    kc, vc = gpu.ops.kv_layout(k_old, v_old, Hkv, hd, max_pos)
+    qkv = H.bits(rng.standard_normal((1, qd + 2 * kvd)))
+    say("attn decode fused", pos, max_pos)
+    out, kc2, vc2 = gpu.ops.attn_decode_rope(qkv, kc, vc, pos, Hq, Hkv, hd, repeats=2)
+    q_rot, kc_ref, vc_ref = gpu.ops.rope_kv_append(qkv, Hq, Hkv, hd, pos, max_pos, kc=kc, vc=vc)
+    assert np.array_equal(kc2, kc_ref) and np.array_equal(vc2, vc_ref)
+    ref = gpu.ops.attn_decode(q_rot[0, :qd], kc_ref, vc_ref, pos + 1, Hq, Hkv, hd)
+    assert np.array_equal(out, ref)
+    q_o = orc.rope(np.ascontiguousarray(qkv[:, :qd]), Hq, hd, pos)
+    k_new = orc.rope(np.ascontiguousarray(qkv[:, qd:qd + kvd]), Hkv, hd, pos)
+    k_all = np.concatenate([k_old, k_new], 0)
+    v_all = np.concatenate([v_old, qkv[:, qd + kvd:]], 0)
+    want = orc.attention(q_o, k_all, v_all, pos, Hq, Hkv, hd).reshape(-1)
+    e = H.mixed_err(out, want)
+    say("  err", e)
+    assert e <= TOL
