@@ -2,8 +2,9 @@
 // softmax over 64-key tiles on v_mfma_f32_32x32x16_f16; the [H,T,T] score
 // tensor of the reference (src/inference/inference.cu:698-947) never exists.
 //
-// One workgroup = one KV head x 32 query rows; wavefront w serves query head
-// kvh*G + w, so the G heads of a group share every K/V tile through LDS.
+// One workgroup = one KV head x 64 query rows (two 32-row tiles); each
+// wavefront serves one query head on one tile, so the G heads of a group and
+// both tiles share every K/V tile through LDS.
 //
 // The kernel computes the transposed problem so that no register shuffles are
 // needed between the two matrix products:
@@ -29,24 +30,37 @@
 #define AP_BQ 32
 #define AP_BKEY 64
 
-template <int HD, int G>
-__global__ __launch_bounds__(G * 64) void attn_prefill_kernel(const half_t *__restrict__ q, int ldq,
-                                                              const half_t *__restrict__ kc,
-                                                              const half_t *__restrict__ vc,
-                                                              half_t *__restrict__ out, int ldo, int T,
-                                                              int pos0, int max_pos) {
-    constexpr int THREADS = G * 64;
+// Workgroup = one KV head x AP_QT query tiles (2, or 1 for groups of 8 heads); wavefront w serves query head
+// kvh*G + w%G on tile w/G, so G*AP_QT wavefronts share every K/V tile.  K/V
+// tiles are double buffered in LDS: tile kt+1 is requested from global memory
+// into registers before the MFMAs of tile kt and written to the other buffer
+// after them (one barrier per tile).
+template <int HD, int G, int AP_QT>
+__global__ __launch_bounds__(G *AP_QT * 64) void attn_prefill_kernel(const half_t *__restrict__ q, int ldq,
+                                                                     const half_t *__restrict__ kc,
+                                                                     const half_t *__restrict__ vc,
+                                                                     half_t *__restrict__ out, int ldo, int T,
+                                                                     int pos0, int max_pos) {
+    constexpr int THREADS = G * AP_QT * 64;
     constexpr int KLD = HD + 8;       // K tile row stride (halves)
     constexpr int VLD = AP_BKEY + 8;  // V^T tile row stride
     constexpr int DS = HD / 16;       // k-steps of the first product
     constexpr int DT = HD / 32;       // 32-row tiles of O^T
-    __shared__ __attribute__((aligned(16))) half_t Ks[AP_BKEY * KLD];
-    __shared__ __attribute__((aligned(16))) half_t Vt[HD * VLD];
+    constexpr int KTILE = AP_BKEY * KLD, VTILE = HD * VLD;
+    constexpr int KCH = AP_BKEY * HD / 8, VCH = HD * AP_BKEY / 8; // 16-byte chunks per tile
+    constexpr int KL = (KCH + THREADS - 1) / THREADS, VL = (VCH + THREADS - 1) / THREADS;
+    extern __shared__ __attribute__((aligned(16))) half_t smem[];
+    half_t *Ks = smem;             // [2][KTILE]
+    half_t *Vt = smem + 2 * KTILE; // [2][VTILE]
 
-    const int qtile = gridDim.x - 1 - blockIdx.x; // longest rows first
+    const int n_qt = (T + AP_BQ - 1) / AP_BQ;
+    const int blk = gridDim.x - 1 - blockIdx.x; // longest rows first
     const int kvh = blockIdx.y;
     const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
-    const int head = kvh * G + wave;
+    const int head = kvh * G + wave % G;
+    int qtile = blk * AP_QT + wave / G;
+    const bool live = qtile < n_qt; // a trailing wavefront without rows still helps with staging
+    if (!live) qtile = n_qt - 1;
     const int n = lane % 32, hb = lane / 32;
     const int q0 = qtile * AP_BQ;
     const int qrow = q0 + n < T ? q0 + n : T - 1;
@@ -63,88 +77,128 @@ __global__ __launch_bounds__(G * 64) void attn_prefill_kernel(const half_t *__re
         for (int e = 0; e < 16; ++e) o[t][e] = 0.f;
     float m_run = -FLT_MAX, l_run = 0.f;
 
-    const int last_q = q0 + AP_BQ - 1 < T - 1 ? q0 + AP_BQ - 1 : T - 1;
-    const int kmax = pos0 + last_q; // last key any row of this tile may see
-    const int n_tiles = kmax / AP_BKEY + 1;
+    const int my_last = (q0 + AP_BQ - 1 < T - 1 ? q0 + AP_BQ - 1 : T - 1) + pos0; // last key this wavefront sees
+    int blk_last_q = (blk + 1) * AP_QT * AP_BQ - 1;
+    if (blk_last_q > T - 1) blk_last_q = T - 1;
+    const int n_tiles = (pos0 + blk_last_q) / AP_BKEY + 1;
     const half_t *kbase = kc + (size_t)kvh * max_pos * HD;
     const half_t *vbase = vc + (size_t)kvh * HD * max_pos;
     const float scale = 1.0f / sqrtf((float)HD);
     const int pm = (n & ~0xC) | ((n & 8) >> 1) | ((n & 4) << 1); // pi(n)
 
+    half8_t rk[KL], rv[VL];
+    auto gload = [&](int key0) {
+#pragma unroll
+        for (int i = 0; i < KL; ++i) {
+            const int c = tid + i * THREADS;
+            if (KCH % THREADS == 0 || c < KCH) rk[i] = load8(kbase + (size_t)(key0 + c / (HD / 8)) * HD + (c % (HD / 8)) * 8);
+        }
+#pragma unroll
+        for (int i = 0; i < VL; ++i) {
+            const int c = tid + i * THREADS;
+            if (VCH % THREADS == 0 || c < VCH)
+                rv[i] = load8(vbase + (size_t)(c / (AP_BKEY / 8)) * max_pos + key0 + (c % (AP_BKEY / 8)) * 8);
+        }
+    };
+    auto sstore = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < KL; ++i) {
+            const int c = tid + i * THREADS;
+            if (KCH % THREADS == 0 || c < KCH) store8(Ks + buf * KTILE + (c / (HD / 8)) * KLD + (c % (HD / 8)) * 8, rk[i]);
+        }
+#pragma unroll
+        for (int i = 0; i < VL; ++i) {
+            const int c = tid + i * THREADS;
+            if (VCH % THREADS == 0 || c < VCH)
+                store8(Vt + buf * VTILE + (c / (AP_BKEY / 8)) * VLD + (c % (AP_BKEY / 8)) * 8, rv[i]);
+        }
+    };
+
+    gload(0);
+    sstore(0);
+    __syncthreads();
     for (int kt = 0; kt < n_tiles; ++kt) {
         const int key0 = kt * AP_BKEY;
-        __syncthreads(); // previous tile fully consumed
-        for (int i = tid; i < AP_BKEY * HD / 8; i += THREADS) {
-            const int r = i / (HD / 8), c = (i % (HD / 8)) * 8;
-            store8(Ks + r * KLD + c, load8(kbase + (size_t)(key0 + r) * HD + c));
+        const int buf = kt & 1;
+        if (kt + 1 < n_tiles) gload(key0 + AP_BKEY);
+        if (live && key0 <= my_last) {
+            const half_t *ks = Ks + buf * KTILE, *vt = Vt + buf * VTILE;
+            // S^T for the two 32-key halves of the tile
+            float16_t st[2];
+#pragma unroll
+            for (int kh = 0; kh < 2; ++kh) {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) st[kh][e] = 0.f;
+                const half_t *kr = ks + (32 * kh + pm) * KLD + 8 * hb;
+#pragma unroll
+                for (int s = 0; s < DS; ++s)
+                    st[kh] = __builtin_amdgcn_mfma_f32_32x32x16_f16(load8(kr + 16 * s), qf[s], st[kh], 0, 0, 0);
+            }
+            // scale, causal mask (only tiles that reach past the first row of this
+            // query tile need it), running max.  accumulator e of half kh is key
+            // key0 + 32*kh + 16*(e/8) + 8*hb + e%8.
+            float mx = -FLT_MAX;
+            if (key0 + AP_BKEY - 1 > pos0 + q0) {
+#pragma unroll
+                for (int kh = 0; kh < 2; ++kh)
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) {
+                        const int key = key0 + 32 * kh + 16 * (e / 8) + 8 * hb + (e % 8);
+                        float sv = st[kh][e] * scale;
+                        sv = key <= qpos ? sv : -FLT_MAX;
+                        st[kh][e] = sv;
+                        mx = fmaxf(mx, sv);
+                    }
+            } else {
+#pragma unroll
+                for (int kh = 0; kh < 2; ++kh)
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) {
+                        const float sv = st[kh][e] * scale;
+                        st[kh][e] = sv;
+                        mx = fmaxf(mx, sv);
+                    }
+            }
+            mx = fmaxf(mx, __shfl_xor(mx, 32));
+            const float m_new = fmaxf(m_run, mx);
+            const float alpha = __expf(m_run - m_new);
+            float psum = 0.f;
+#pragma unroll
+            for (int kh = 0; kh < 2; ++kh)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    const float sv = st[kh][e];
+                    const float p = sv == -FLT_MAX ? 0.f : __expf(sv - m_new);
+                    st[kh][e] = p;
+                    psum += p;
+                }
+            psum += __shfl_xor(psum, 32);
+            l_run = l_run * alpha + psum;
+            m_run = m_new;
+#pragma unroll
+            for (int t = 0; t < DT; ++t)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) o[t][e] *= alpha;
+
+            // O^T += V^T . P^T, four 16-key steps
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                half8_t pb;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) pb[j] = (half_t)st[u / 2][8 * (u % 2) + j];
+#pragma unroll
+                for (int t = 0; t < DT; ++t) {
+                    half8_t vf = load8(vt + (32 * t + n) * VLD + 16 * u + 8 * hb);
+                    o[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, pb, o[t], 0, 0, 0);
+                }
+            }
         }
-        for (int i = tid; i < HD * AP_BKEY / 8; i += THREADS) {
-            const int d = i / (AP_BKEY / 8), c = (i % (AP_BKEY / 8)) * 8;
-            store8(Vt + d * VLD + c, load8(vbase + (size_t)d * max_pos + key0 + c));
-        }
+        if (kt + 1 < n_tiles) sstore(buf ^ 1);
         __syncthreads();
-
-        // S^T for the two 32-key halves of the tile
-        float16_t st[2];
-#pragma unroll
-        for (int kh = 0; kh < 2; ++kh) {
-#pragma unroll
-            for (int e = 0; e < 16; ++e) st[kh][e] = 0.f;
-            const half_t *kr = Ks + (32 * kh + pm) * KLD + 8 * hb;
-#pragma unroll
-            for (int s = 0; s < DS; ++s)
-                st[kh] = __builtin_amdgcn_mfma_f32_32x32x16_f16(load8(kr + 16 * s), qf[s], st[kh], 0, 0, 0);
-        }
-        // scale, causal mask, running max.  accumulator e of half kh is key
-        // key0 + 32*kh + 16*(e/8) + 8*hb + e%8.
-        float mx = -FLT_MAX;
-#pragma unroll
-        for (int kh = 0; kh < 2; ++kh)
-#pragma unroll
-            for (int e = 0; e < 16; ++e) {
-                const int key = key0 + 32 * kh + 16 * (e / 8) + 8 * hb + (e % 8);
-                float s = st[kh][e] * scale;
-                s = key <= qpos ? s : -FLT_MAX;
-                st[kh][e] = s;
-                mx = fmaxf(mx, s);
-            }
-        mx = fmaxf(mx, __shfl_xor(mx, 32));
-        const float m_new = fmaxf(m_run, mx);
-        const float alpha = __expf(m_run - m_new);
-        float psum = 0.f;
-#pragma unroll
-        for (int kh = 0; kh < 2; ++kh)
-#pragma unroll
-            for (int e = 0; e < 16; ++e) {
-                const float s = st[kh][e];
-                const float p = s == -FLT_MAX ? 0.f : __expf(s - m_new);
-                st[kh][e] = p;
-                psum += p;
-            }
-        psum += __shfl_xor(psum, 32);
-        l_run = l_run * alpha + psum;
-        m_run = m_new;
-#pragma unroll
-        for (int t = 0; t < DT; ++t)
-#pragma unroll
-            for (int e = 0; e < 16; ++e) o[t][e] *= alpha;
-
-        // O^T += V^T . P^T, four 16-key steps
-#pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            half8_t pb;
-#pragma unroll
-            for (int j = 0; j < 8; ++j) pb[j] = (half_t)st[u / 2][8 * (u % 2) + j];
-#pragma unroll
-            for (int t = 0; t < DT; ++t) {
-                half8_t vf = load8(Vt + (32 * t + n) * VLD + 16 * u + 8 * hb);
-                o[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, pb, o[t], 0, 0, 0);
-            }
-        }
     }
 
     // O^T lane l: query q0 + l%32, dims 32t + 8*(e/4) + 4*(l/32) + e%4
-    if (q0 + n < T) {
+    if (live && q0 + n < T) {
         const float inv = 1.0f / l_run;
         half_t *orow = out + (size_t)(q0 + n) * ldo + (size_t)head * HD;
 #pragma unroll
@@ -162,8 +216,17 @@ __global__ __launch_bounds__(G * 64) void attn_prefill_kernel(const half_t *__re
 template <int HD, int G>
 static int launch_prefill(const half_t *q, int ldq, const half_t *kc, const half_t *vc, half_t *out, int ldo,
                           int T, int pos0, int n_kv_heads, int max_pos, hipStream_t s) {
-    dim3 grid((T + AP_BQ - 1) / AP_BQ, n_kv_heads);
-    attn_prefill_kernel<HD, G><<<grid, dim3(G * 64), 0, s>>>(q, ldq, kc, vc, out, ldo, T, pos0, max_pos);
+    constexpr int AP_QT = G >= 8 ? 1 : 2; // 32-row query tiles per workgroup (at most 8 wavefronts)
+    const int n_qt = (T + AP_BQ - 1) / AP_BQ;
+    dim3 grid((n_qt + AP_QT - 1) / AP_QT, n_kv_heads);
+    const size_t smem = sizeof(half_t) * 2 * ((size_t)AP_BKEY * (HD + 8) + (size_t)HD * (AP_BKEY + 8));
+    auto kern = attn_prefill_kernel<HD, G, AP_QT>;
+    static bool attr_set = false;
+    if (!attr_set && smem > 48 * 1024) {
+        LLM_HIP_CHECK(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+        attr_set = true;
+    }
+    kern<<<grid, dim3(G * AP_QT * 64), smem, s>>>(q, ldq, kc, vc, out, ldo, T, pos0, max_pos);
     LLM_LAUNCH_CHECK("attn_prefill_kernel");
     return LLM_OK;
 }

@@ -127,17 +127,26 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_kernel(const half_t *__res
     half_t *As = lds;                                    // [2][BM][GEMM_LD]
     half_t *Bs = lds + 2 * BM * GEMM_LD;                 // [2][NB][BN][GEMM_LD]
 
-    // XCD-aware tile order: consecutive workgroup ids land on different XCDs
-    // (8 of them), so give each XCD a contiguous run of tiles, and walk the
-    // tiles of a run down M first so neighbours share the weight (B) tile in
-    // that XCD's L2.
+    // XCD-aware tile order.  Consecutive workgroup ids land on different XCDs
+    // (8 of them, each with its own L2), so each XCD first gets a contiguous
+    // run of logical tiles; inside a run the tiles walk GROUP_M rows of M for
+    // every N column, so the ~32 tiles an XCD works on at a time form a compact
+    // 8 x 4 block that shares its A rows and B rows through that XCD's L2.
     const int nblk = tiles_m * tiles_n;
     int bid = blockIdx.x;
     {
         const int per = nblk / 8;
         if (per > 0 && bid < per * 8) bid = (bid % 8) * per + bid / 8;
     }
-    const int tm = bid % tiles_m, tn = bid / tiles_m;
+#ifndef GEMM_GROUP_M
+#define GEMM_GROUP_M 8
+#endif
+    constexpr int GROUP_M = GEMM_GROUP_M;
+    const int group = bid / (GROUP_M * tiles_n);
+    const int first_m = group * GROUP_M;
+    const int gsz = tiles_m - first_m < GROUP_M ? tiles_m - first_m : GROUP_M;
+    const int tm = first_m + (bid % (GROUP_M * tiles_n)) % gsz;
+    const int tn = (bid % (GROUP_M * tiles_n)) / gsz;
     const int m0 = tm * BM, n0 = tn * BN;
 
     const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
@@ -173,57 +182,84 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_kernel(const half_t *__res
 #pragma unroll
                 for (int e = 0; e < 16; ++e) acc[b][i][j][e] = 0.f;
 
-    half8_t ra[A_LOADS], rb[NB][B_LOADS];
-    auto gload = [&](int k0) {
+    // Global loads run DEPTH k-tiles ahead of the MFMAs through DEPTH register
+    // sets: tile kt+DEPTH is requested at the top of iteration kt, and tile kt+1
+    // (requested DEPTH iterations earlier) is written to the other LDS buffer at
+    // the bottom, so a trip to HBM has DEPTH iterations of matrix work to hide
+    // behind.  One wavefront per SIMD (4-wave tiles) has the registers for two.
+    constexpr int DEPTH = (WGM * WGN <= 4) ? 2 : 1;
+    half8_t ra[DEPTH][A_LOADS], rb[DEPTH][NB][B_LOADS];
+    auto gload = [&](int set, int k0) {
 #pragma unroll
-        for (int i = 0; i < A_LOADS; ++i) ra[i] = load8(ag[i] + k0);
+        for (int i = 0; i < A_LOADS; ++i) ra[set][i] = load8(ag[i] + k0);
 #pragma unroll
         for (int b = 0; b < NB; ++b)
 #pragma unroll
-            for (int i = 0; i < B_LOADS; ++i) rb[b][i] = load8(bg[b][i] + k0);
+            for (int i = 0; i < B_LOADS; ++i) rb[set][b][i] = load8(bg[b][i] + k0);
     };
-    auto sstore = [&](int buf) {
+    auto sstore = [&](int set, int buf) {
         half_t *a = As + buf * BM * GEMM_LD;
 #pragma unroll
-        for (int i = 0; i < A_LOADS; ++i) store8(a + (srow + i * ROWS_PER_PASS) * GEMM_LD + scol, ra[i]);
+        for (int i = 0; i < A_LOADS; ++i) store8(a + (srow + i * ROWS_PER_PASS) * GEMM_LD + scol, ra[set][i]);
 #pragma unroll
         for (int b = 0; b < NB; ++b) {
             half_t *bb = Bs + (buf * NB + b) * BN * GEMM_LD;
 #pragma unroll
-            for (int i = 0; i < B_LOADS; ++i) store8(bb + (srow + i * ROWS_PER_PASS) * GEMM_LD + scol, rb[b][i]);
+            for (int i = 0; i < B_LOADS; ++i) store8(bb + (srow + i * ROWS_PER_PASS) * GEMM_LD + scol, rb[set][b][i]);
         }
     };
-
-    const int nk = K / GEMM_BK;
-    gload(0);
-    sstore(0);
-    __syncthreads();
-
     const int frow = lane % 32, fk = (lane / 32) * 8;
-    for (int kt = 0; kt < nk; ++kt) {
-        const int buf = kt & 1;
-        if (kt + 1 < nk) gload((kt + 1) * GEMM_BK);
+    // Fragments of k-step ks+1 are read from LDS while the MFMAs of k-step ks
+    // run (two fragment register sets), so LDS latency sits behind matrix work.
+    auto compute = [&](int buf) {
         const half_t *a = As + buf * BM * GEMM_LD + (wm * TM + frow) * GEMM_LD + fk;
+        const half_t *bp[NB];
+#pragma unroll
+        for (int b = 0; b < NB; ++b) bp[b] = Bs + (buf * NB + b) * BN * GEMM_LD + (wn * TN + frow) * GEMM_LD + fk;
+        half8_t af[2][FM], bf[2][NB][FN];
+        auto lfrag = [&](int set, int ks) {
+#pragma unroll
+            for (int i = 0; i < FM; ++i) af[set][i] = load8(a + i * 32 * GEMM_LD + ks * 16);
+#pragma unroll
+            for (int b = 0; b < NB; ++b)
+#pragma unroll
+                for (int j = 0; j < FN; ++j) bf[set][b][j] = load8(bp[b] + j * 32 * GEMM_LD + ks * 16);
+        };
+        lfrag(0, 0);
 #pragma unroll
         for (int ks = 0; ks < GEMM_BK / 16; ++ks) {
-            half8_t af[FM];
+            const int cur = ks & 1;
+            if (ks + 1 < GEMM_BK / 16) lfrag(cur ^ 1, ks + 1);
+            __builtin_amdgcn_sched_barrier(0); // keep the LDS reads ahead of this step's MFMAs
 #pragma unroll
-            for (int i = 0; i < FM; ++i) af[i] = load8(a + i * 32 * GEMM_LD + ks * 16);
-#pragma unroll
-            for (int b = 0; b < NB; ++b) {
-                const half_t *bp = Bs + (buf * NB + b) * BN * GEMM_LD + (wn * TN + frow) * GEMM_LD + fk;
-                half8_t bf[FN];
-#pragma unroll
-                for (int j = 0; j < FN; ++j) bf[j] = load8(bp + j * 32 * GEMM_LD + ks * 16);
+            for (int b = 0; b < NB; ++b)
 #pragma unroll
                 for (int i = 0; i < FM; ++i)
 #pragma unroll
                     for (int j = 0; j < FN; ++j)
-                        acc[b][i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf[j], acc[b][i][j], 0, 0, 0);
-            }
+                        acc[b][i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[cur][i], bf[cur][b][j], acc[b][i][j], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
         }
-        if (kt + 1 < nk) sstore(buf ^ 1);
+    };
+
+    const int nk = K / GEMM_BK;
+    gload(0, 0);
+    sstore(0, 0);
+    if (DEPTH == 2 && nk > 1) gload(DEPTH - 1, GEMM_BK);
+    __syncthreads();
+    // unrolled by two so that register-set and LDS-buffer indices are constants:
+    // iteration kt uses LDS buffer kt%2; with DEPTH 2, tile kt+1 sits in register set (kt+1)%2
+    for (int kt = 0; kt < nk; kt += 2) {
+        if (kt + DEPTH < nk) gload(0, (kt + DEPTH) * GEMM_BK);
+        compute(0);
+        if (kt + 1 < nk) sstore(DEPTH - 1, 1);
         __syncthreads();
+        if (kt + 1 < nk) {
+            if (kt + 1 + DEPTH < nk) gload(DEPTH - 1, (kt + 1 + DEPTH) * GEMM_BK);
+            compute(1);
+            if (kt + 2 < nk) sstore(0, 0);
+            __syncthreads();
+        }
     }
 
     // epilogue: D lane l -> col l%32, rows 8*(e/4) + 4*(l/32) + e%4
@@ -296,7 +332,7 @@ int llm_linear(const uint16_t *x, int ldx, const uint16_t *w, const uint16_t *re
     }
     if (T <= 64 || N < 256) return gemm_launch<64, 64, 2, 2, 1>(xp, ldx, wp, nullptr, rp, ldr, op, ldo, T, N, K, s);
     if (T <= 128) return gemm_launch<128, 128, 2, 2, 1>(xp, ldx, wp, nullptr, rp, ldr, op, ldo, T, N, K, s);
-    return gemm_launch<256, 256, 2, 2, 1>(xp, ldx, wp, nullptr, rp, ldr, op, ldo, T, N, K, s);
+    return gemm_launch<256, 256, 4, 2, 1>(xp, ldx, wp, nullptr, rp, ldr, op, ldo, T, N, K, s);
 }
 
 int llm_linear_swiglu(const uint16_t *x, int ldx, const uint16_t *wgate, const uint16_t *wup, uint16_t *out,
@@ -317,7 +353,7 @@ int llm_linear_swiglu(const uint16_t *x, int ldx, const uint16_t *wgate, const u
     }
     if (T <= 64 || N < 256) return gemm_launch<64, 64, 2, 2, 2>(xp, ldx, gp, up, nullptr, 0, op, ldo, T, N, K, s);
     if (T <= 128) return gemm_launch<128, 64, 2, 2, 2>(xp, ldx, gp, up, nullptr, 0, op, ldo, T, N, K, s);
-    return gemm_launch<256, 128, 2, 2, 2>(xp, ldx, gp, up, nullptr, 0, op, ldo, T, N, K, s);
+    return gemm_launch<256, 128, 4, 2, 2>(xp, ldx, gp, up, nullptr, 0, op, ldo, T, N, K, s);
 }
 
 int llm_norm_linear(const uint16_t *x, const uint16_t *gain, double eps, const uint16_t *w, uint16_t *out, int N, int K,
