@@ -142,6 +142,12 @@ int llama3_generate(Llama3 *m, CudaCache *c, const int *prompt, int n_prompt, in
  * llama3_read_logits copies the fp16 logits of the last processed row. */
 void llama3_set_hidden_trace(CudaCache *c, llm_half *hidden);
 void llama3_read_logits(CudaCache *c, llm_half *logits);
+/* Teacher forcing for per-layer parity: during the next prefill/decode call,
+ * layer l >= 1 starts from rows hidden[l-1] ([n_layers][n][d_model] fp16 bits,
+ * host memory, e.g. another implementation's trace) instead of this engine's
+ * own layer l-1 output, so each layer is compared on identical input and
+ * rounding differences do not compound across layers. */
+void llama3_set_hidden_inject(CudaCache *c, const llm_half *hidden);
 
 /* Choose between one hipGraph replay per decode step (1, default) and plain
  * stream launches (0). */

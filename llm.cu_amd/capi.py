@@ -145,6 +145,7 @@ HOST_ABI = {
     "llama3_generate": (_i, [_LP, _CP, C.POINTER(_i), _i, _i, C.POINTER(_i), C.POINTER(GenStats)]),
     "llama3_set_hidden_trace": (None, [_CP, _vp]),
     "llama3_read_logits": (None, [_CP, _vp]),
+    "llama3_set_hidden_inject": (None, [_CP, _vp]),
     "llama3_set_use_graph": (None, [_CP, _i]),
     "llama3_set_error_handler": (None, [_vp]),
     "seeded_normal_bf16": (None, [_u64, _u64, _sz, C.c_float, _vp]),

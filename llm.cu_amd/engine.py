@@ -113,15 +113,24 @@ class Engine:
         lib().llama3_set_hidden_trace(self.cache, buf.ctypes.data)
         return buf
 
-    def prefill(self, tokens, want_hidden=False):
+    def prefill(self, tokens, want_hidden=False, inject=None):
+        """inject: [n_layers, n, d] uint16 hidden states; layer l >= 1 starts from inject[l-1]."""
         tokens = np.ascontiguousarray(tokens, dtype=np.int32)
         hidden = self._trace(tokens.size) if want_hidden else None
+        if inject is not None:
+            inject = np.ascontiguousarray(inject, dtype=np.uint16)
+            assert inject.shape == (self.cfg.n_layers, tokens.size, self.cfg.d_model)
+            lib().llama3_set_hidden_inject(self.cache, inject.ctypes.data)
         tok = lib().llama3_prefill(self.model.handle, self.cache,
                                    tokens.ctypes.data_as(C.POINTER(C.c_int)), tokens.size)
         return tok, hidden
 
-    def decode(self, token, want_hidden=False):
+    def decode(self, token, want_hidden=False, inject=None):
         hidden = self._trace(1) if want_hidden else None
+        if inject is not None:
+            inject = np.ascontiguousarray(inject, dtype=np.uint16)
+            assert inject.shape == (self.cfg.n_layers, 1, self.cfg.d_model)
+            lib().llama3_set_hidden_inject(self.cache, inject.ctypes.data)
         tok = lib().llama3_decode(self.model.handle, self.cache, int(token))
         return tok, hidden
 

@@ -43,6 +43,9 @@ struct Engine {
     llm_half *trace_dev = nullptr;
     size_t trace_rows = 0;
     llm_half *trace_host = nullptr;
+    const llm_half *inject_host = nullptr; // teacher forcing: layer l >= 1 starts from these rows
+    llm_half *inject_dev = nullptr;
+    size_t inject_rows = 0;
     std::vector<int> tokens; // ids whose K/V are cached
     int pos = 0;
     bool use_graph = true;
@@ -101,7 +104,7 @@ void check_shapes(const Llama3 *m, const ModelConfig &c) {
 
 // Issues one pass over T rows on the engine's stream.  With dev_pos the row
 // position comes from *d_pos (T must be 1): that form is what gets captured.
-void issue_pass(Engine *e, const Llama3 *m, int T, int pos0, bool dev_pos, bool trace) {
+void issue_pass(Engine *e, const Llama3 *m, int T, int pos0, bool dev_pos, bool trace, bool inject = false) {
     const ModelConfig &c = e->cfg;
     const int d = c.d_model, hd = c.head_dim, Hq = c.n_heads, Hkv = c.n_kv_heads, F = c.ffn_dim;
     const int qd = Hq * hd, kvd = Hkv * hd, QKV = e->qkv_dim;
@@ -118,6 +121,9 @@ void issue_pass(Engine *e, const Llama3 *m, int T, int pos0, bool dev_pos, bool 
         for (int l = 0; l < c.n_layers; ++l) {
             const LayerW w = layer_w(m, l);
             llm_half *kc = e->kc + (size_t)l * e->kv_layer_elems, *vc = e->vc + (size_t)l * e->kv_layer_elems;
+            if (inject && l > 0)
+                llama3_check(llm_memcpy_d2d(e->x, e->inject_dev + (size_t)(l - 1) * d, sizeof(llm_half) * (size_t)d, s),
+                             "inject copy");
             if (w.wk == w.wq + (size_t)qd * d && w.wv == w.wk + (size_t)kvd * d) {
                 llama3_check(llm_norm_linear(e->x, w.in_ln, c.rms_eps, w.wq, e->qkv, QKV, d, s), "llm_norm_linear(qkv)");
             } else {
@@ -141,6 +147,10 @@ void issue_pass(Engine *e, const Llama3 *m, int T, int pos0, bool dev_pos, bool 
         for (int l = 0; l < c.n_layers; ++l) {
             const LayerW w = layer_w(m, l);
             llm_half *kc = e->kc + (size_t)l * e->kv_layer_elems, *vc = e->vc + (size_t)l * e->kv_layer_elems;
+            if (inject && l > 0)
+                llama3_check(llm_memcpy_d2d(e->x, e->inject_dev + (size_t)(l - 1) * T * d,
+                                            sizeof(llm_half) * (size_t)T * d, s),
+                             "inject copy");
             llama3_check(llm_rmsnorm(e->x, w.in_ln, e->xn, T, d, c.rms_eps, s), "llm_rmsnorm");
             if (w.wk == w.wq + (size_t)qd * d && w.wv == w.wk + (size_t)kvd * d) {
                 llama3_check(llm_linear(e->xn, d, w.wq, nullptr, 0, e->qkv, QKV, T, QKV, d, s), "llm_linear(qkv)");
@@ -197,7 +207,17 @@ int run_pass(Engine *e, const Llama3 *m, const int *tokens, int n) {
             e->trace_rows = need;
         }
     }
-    issue_pass(e, m, n, e->pos, false, trace);
+    const bool inject = e->inject_host != nullptr;
+    if (inject) {
+        size_t need = (size_t)c.n_layers * n * c.d_model;
+        if (need > e->inject_rows) {
+            if (e->inject_dev) llm_free(e->inject_dev);
+            e->inject_dev = dmalloc<llm_half>(need, "llm_malloc(inject)");
+            e->inject_rows = need;
+        }
+        llama3_check(llm_memcpy_h2d(e->inject_dev, e->inject_host, sizeof(llm_half) * need, s), "H2D inject");
+    }
+    issue_pass(e, m, n, e->pos, false, trace, inject);
     int32_t tok = -1;
     llama3_check(llm_memcpy_d2h(&tok, e->d_token, sizeof(int32_t), s), "D2H token");
     if (trace)
@@ -205,6 +225,7 @@ int run_pass(Engine *e, const Llama3 *m, const int *tokens, int n) {
                      "D2H trace");
     llama3_check(llm_stream_sync(s), "stream sync");
     e->trace_host = nullptr;
+    e->inject_host = nullptr;
     e->tokens.insert(e->tokens.end(), tokens, tokens + n);
     e->pos += n;
     return (int)tok;
@@ -302,7 +323,7 @@ extern "C" void free_cache(CudaCache *C) {
         llm_stream_sync(e->stream);
         drop_graph(e);
         void *bufs[] = {e->x, e->xn, e->qkv, e->attn, e->ffn, e->logits, e->kc, e->vc, e->rope_table,
-                        e->d_tokens, e->d_pos, e->d_token, e->ws_attn, e->ws_lm, e->trace_dev};
+                        e->d_tokens, e->d_pos, e->d_token, e->ws_attn, e->ws_lm, e->trace_dev, e->inject_dev};
         for (void *b : bufs) llm_free(b);
         for (auto ev : e->ev) llm_event_destroy(ev);
         llm_stream_destroy(e->stream);
@@ -345,7 +366,7 @@ extern "C" int llama3_prefill(Llama3 *m, CudaCache *C, const int *tokens, int n)
 
 extern "C" int llama3_decode(Llama3 *m, CudaCache *C, int token) {
     Engine *e = eng(C);
-    if (e->trace_host) return run_pass(e, m, &token, 1);
+    if (e->trace_host || e->inject_host) return run_pass(e, m, &token, 1);
     const ModelConfig &c = e->cfg;
     if (e->pos + 1 > c.max_pos) llama3_fail("sequence of %d tokens exceeds max_pos %d", e->pos + 1, c.max_pos);
     if (token < 0 || token >= c.vocab) llama3_fail("token id %d outside the vocabulary", token);
@@ -408,6 +429,8 @@ extern "C" int llama3_generate(Llama3 *m, CudaCache *C, const int *prompt, int n
 }
 
 extern "C" void llama3_set_hidden_trace(CudaCache *C, llm_half *hidden) { eng(C)->trace_host = hidden; }
+
+extern "C" void llama3_set_hidden_inject(CudaCache *C, const llm_half *hidden) { eng(C)->inject_host = hidden; }
 
 extern "C" void llama3_read_logits(CudaCache *C, llm_half *logits) {
     Engine *e = eng(C);

@@ -215,8 +215,8 @@ void orc_add(uint16_t *x, const uint16_t *res, size_t n) {
 /* ------------------------------------------------------------------ */
 #define TBLK 64
 
-static void matmul_raw(const float *x, size_t ldx, const uint16_t *w, int T, int N, int K,
-                       float *out, size_t ldo, int r16) {
+static void matmul_raw_ord(const float *x, size_t ldx, const uint16_t *w, int T, int N, int K,
+                           float *out, size_t ldo, int r16, int rev) {
     if (T == 1) {
 #pragma omp parallel
         {
@@ -231,7 +231,8 @@ static void matmul_raw(const float *x, size_t ldx, const uint16_t *w, int T, int
                     const float *w0 = wr, *w1 = wr + K, *w2 = wr + 2 * (size_t)K, *w3 = wr + 3 * (size_t)K,
                                 *w4 = wr + 4 * (size_t)K, *w5 = wr + 5 * (size_t)K,
                                 *w6 = wr + 6 * (size_t)K, *w7 = wr + 7 * (size_t)K;
-                    for (int k = 0; k < K; ++k) {
+                    for (int kk = 0; kk < K; ++kk) {
+                        const int k = rev ? K - 1 - kk : kk;
                         float xv = x[k];
                         a0 += xv * w0[k]; a1 += xv * w1[k]; a2 += xv * w2[k]; a3 += xv * w3[k];
                         a4 += xv * w4[k]; a5 += xv * w5[k]; a6 += xv * w6[k]; a7 += xv * w7[k];
@@ -242,7 +243,10 @@ static void matmul_raw(const float *x, size_t ldx, const uint16_t *w, int T, int
                     for (int r = 0; r < nr; ++r) {
                         float a = 0.f;
                         const float *wp = wr + (size_t)r * K;
-                        for (int k = 0; k < K; ++k) a += x[k] * wp[k];
+                        for (int kk = 0; kk < K; ++kk) {
+                            const int k = rev ? K - 1 - kk : kk;
+                            a += x[k] * wp[k];
+                        }
                         out[n0 + r] = a;
                     }
                 } else {
@@ -275,7 +279,8 @@ static void matmul_raw(const float *x, size_t ldx, const uint16_t *w, int T, int
                 widen(w + (size_t)n * K, wr, K);
                 float acc[TBLK];
                 for (int t = 0; t < TBLK; ++t) acc[t] = 0.f;
-                for (int k = 0; k < K; ++k) {
+                for (int kk = 0; kk < K; ++kk) {
+                    const int k = rev ? K - 1 - kk : kk;
                     float wk = wr[k];
                     const float *xr = xT + (size_t)k * TBLK;
 #pragma omp simd
@@ -287,6 +292,14 @@ static void matmul_raw(const float *x, size_t ldx, const uint16_t *w, int T, int
         }
     }
     free(xT);
+}
+
+/* ORC_REF16_REV sums k downwards: a second, equally valid fp32 order, used only to
+ * measure how far rounding-order differences alone move the hidden states. */
+static int g_rev_k = 0;
+static void matmul_raw(const float *x, size_t ldx, const uint16_t *w, int T, int N, int K,
+                       float *out, size_t ldo, int r16) {
+    matmul_raw_ord(x, ldx, w, T, N, K, out, ldo, r16, g_rev_k);
 }
 
 void orc_linear(const uint16_t *x, const uint16_t *w, int T, int N, int K, uint16_t *out) {
@@ -665,8 +678,10 @@ static int forward_rows(const orc_config *c, const orc_weights *w, int r16, floa
 int orc_model_forward(orc_model *m, const int32_t *tokens, int n_new, uint16_t *hidden_out,
                       uint16_t *logits_out) {
     if (n_new <= 0 || m->pos + n_new > m->cfg.max_pos) return -1;
-    int tok = forward_rows(&m->cfg, &m->w, m->mode == ORC_REF16, m->kc, m->vc, tokens, n_new,
+    g_rev_k = m->mode == ORC_REF16_REV;
+    int tok = forward_rows(&m->cfg, &m->w, m->mode != ORC_FP32, m->kc, m->vc, tokens, n_new,
                            m->pos, hidden_out, logits_out);
+    g_rev_k = 0;
     m->pos += n_new;
     return tok;
 }

@@ -13,6 +13,10 @@
  *   ORC_FP32   same graph, no intermediate rounding, free accumulation order,
  *              OpenMP over rows/heads -- the timed "fp32 forward" CPU baseline.
  *
+ *   ORC_REF16_REV  ORC_REF16 with every projection summed over k downwards: the same
+ *              arithmetic in another legal fp32 order.  Not a parity target; it
+ *              measures how much of a deviation is summation order alone.
+ *
  * Every function cites the reference lines it restates (paths under
  * src/ of abhisheknair10/LLM.cu).
  */
@@ -26,7 +30,7 @@
 extern "C" {
 #endif
 
-enum { ORC_REF16 = 0, ORC_FP32 = 1 };
+enum { ORC_REF16 = 0, ORC_FP32 = 1, ORC_REF16_REV = 2 };
 
 typedef struct {
     int n_layers;

@@ -16,6 +16,7 @@ _LIB_PATH = os.path.join(_HERE, "liboracle.so")
 
 ORC_REF16 = 0
 ORC_FP32 = 1
+ORC_REF16_REV = 2
 
 
 class OrcConfig(C.Structure):

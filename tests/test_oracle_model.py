@@ -54,6 +54,23 @@ def test_ref16_and_fp32_agree_within_tolerance(pkg):
     assert ta == tb
 
 
+def test_reversed_order_mode_is_a_reordering_only(pkg):
+    """ORC_REF16_REV sums every projection over k downwards: close to ORC_REF16 (same terms), not
+    identical (fp32 addition is not associative), and the switch does not leak into later models."""
+    cfg, cd, w, prompt = _setup(pkg)
+    a = orc.Model(cd, w, orc.ORC_REF16)
+    r = orc.Model(cd, w, orc.ORC_REF16_REV)
+    ta, ha, la = a.forward(prompt, want_hidden=True)
+    tr, hr, lr = r.forward(prompt, want_hidden=True)
+    assert H.mixed_err(ha, hr) < H.TOL and H.mixed_err(la, lr) < H.TOL
+    assert not np.array_equal(ha, hr)
+    assert ta == tr
+    # the mode must not leak into later ORC_REF16 models
+    a2 = orc.Model(cd, w, orc.ORC_REF16)
+    _, ha2, _ = a2.forward(prompt, want_hidden=True)
+    assert np.array_equal(ha, ha2)
+
+
 def test_golden_fixture(pkg):
     """tests/golden/tiny_seed1234.json was written by tests/golden/make_tiny_fixture.py
     from this oracle; it travels to the GPU box and pins the oracle build there
