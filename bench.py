@@ -27,6 +27,12 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK = 8.0e12          # B/s, MI355X HBM3E
+# HBM bytes one launch of the gate/up SwiGLU GEMV moves, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE
+# (two runs of this script), each scaled by the same counter's reading for the calibration copy of
+# kernel_roofline() (FETCH_SIZE reads 0.5001 of the bytes a plain streaming pass fetches on this part,
+# WRITE_SIZE 1.0000): 234,985,724 fetched + 114,697 written; profiles/gemv_swiglu_hbm_traffic.md holds
+# the counter readings.
+GEMV_SWIGLU_TRAFFIC_BYTES = 235100421
 MFMA_F16_PEAK = 2.5e15     # flop/s, MI355X dense fp16
 
 
@@ -193,11 +199,22 @@ def kernel_roofline(pkg, model, cfg):
             pkg.capi.check(lib.llm_linear_swiglu(x.ptr, d, wg[l], wu[l], out.ptr, F, 1, F, d, stream))
 
     ms = timer.time(issue, iters=8, warmup=2) / cfg.n_layers
+    # One plain streaming pass of known size (2^26 elements: 128 MiB read, 128 MiB written) as the
+    # calibration dispatch for the FETCH_SIZE / WRITE_SIZE counters; it is the last bf16_to_fp16_kernel
+    # dispatch of the run.
+    n_cal = 1 << 26
+    cal_in = pkg.capi.DevBuf((n_cal,), np.uint16)
+    cal_out = pkg.capi.DevBuf((n_cal,), np.uint16)
+    pkg.capi.check(lib.llm_fill_zero(cal_in.ptr, n_cal * 2, None))
+    pkg.capi.check(lib.llm_bf16_to_fp16(cal_in.ptr, cal_out.ptr, n_cal, None))
+    pkg.capi.sync()
+    cal_in.free()
+    cal_out.free()
     alg = 2 * 2 * F * d + 2 * d + 2 * F  # two weight matrices + activation in + result out
     achieved = alg / (ms * 1e-3)
     return {"kernel": "gemv_swiglu_kernel (gate+up, N=14336, K=4096, T=1)", "bound": "hbm",
             "achieved": achieved / 1e9, "peak": HBM_PEAK / 1e9, "unit": "GB/s", "frac": achieved / HBM_PEAK,
-            "traffic": None, "avg_launch_us": ms * 1e3, "algorithmic_bytes_per_launch": alg,
+            "traffic": GEMV_SWIGLU_TRAFFIC_BYTES, "avg_launch_us": ms * 1e3, "algorithmic_bytes_per_launch": alg,
             "launches_timed": 8 * cfg.n_layers}
 
 
