@@ -301,6 +301,220 @@ static int gemm_launch(const half_t *x, int ldx, const half_t *w, const half_t *
 }
 
 // ---------------------------------------------------------------------------
+// large-T MFMA GEMM: tiles go from global memory straight into LDS
+// ---------------------------------------------------------------------------
+// No register staging: every wavefront issues global_load_lds (16 B per lane, 1 KB per instruction,
+// landing contiguously in LDS), STAGES buffers deep, and waits with an explicit vmcnt so that loads
+// stay in flight across workgroup barriers.  Because a wave instruction fills 16 consecutive 64-byte
+// rows, the row padding of the kernel above is not available; instead lane l fetches global 16-byte
+// chunk (l%4) ^ ((row>>2)&3) of its row, so that the 16 lanes an LDS read serves per cycle (16 rows,
+// same logical chunk) fall into 16 different 16-byte bank groups.
+#define DMA_BK 32
+#define DMA_GP(p) ((const __attribute__((address_space(1))) void *)(p))
+#define DMA_LP(p) ((__attribute__((address_space(3))) void *)(p))
+
+template <int N> __device__ __forceinline__ void dma_wait_barrier() {
+    // vmcnt(N): all but the newest N of this wave's loads have landed; then the workgroup barrier.
+    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(N) : "memory");
+}
+
+// 256 x (WGN*128) macro-tile, WGN*4 wavefronts each owning 64 x 128 of it (NB = 2: 64 columns of gate and
+// the same 64 of up), BK = 32, STAGES LDS buffers filled by direct global->LDS loads.
+// PREF: read the next tile's first fragments before the barrier (needs tiles kt and kt+1 landed at
+// barrier kt, so loads run STAGES-2 iterations ahead); otherwise loads run STAGES-1 ahead.
+template <int NB, int WGN, int STAGES, bool PREF, int OCC>
+__global__ __launch_bounds__(WGN * 256, OCC) void gemm_dma_kernel(const half_t *__restrict__ x, int ldx,
+                                                               const half_t *__restrict__ w, const half_t *__restrict__ w2,
+                                                               const half_t *res, int ldr, half_t *out, int ldo, int T, int N, int K,
+                                                               int tiles_m, int tiles_n) {
+    constexpr int NWAVES = 4 * WGN;
+    constexpr int BM = 256, BROWS = WGN * 128; // B rows in a stage (both matrices when NB = 2)
+    constexpr int BN = BROWS / NB;             // output columns per tile
+    constexpr int FM = 2, FN = 4 / NB;
+    constexpr int STAGE_HALVES = (BM + BROWS) * DMA_BK;
+    constexpr int LPT = (BM + BROWS) / 16 / NWAVES; // load instructions per wave per tile
+    constexpr int AHEAD = PREF ? STAGES - 2 : STAGES - 1;
+    static_assert(16 % NWAVES == 0 || NWAVES == 8, "loader split");
+    extern __shared__ __attribute__((aligned(16))) half_t lds[];
+
+    const int nblk = tiles_m * tiles_n;
+    int bid = blockIdx.x;
+    {
+        const int per = nblk / 8;
+        if (per > 0 && bid < per * 8) bid = (bid % 8) * per + bid / 8;
+    }
+    constexpr int GROUP_M = 8;
+    const int group = bid / (GROUP_M * tiles_n);
+    const int first_m = group * GROUP_M;
+    const int gsz = tiles_m - first_m < GROUP_M ? tiles_m - first_m : GROUP_M;
+    const int tm = first_m + (bid % (GROUP_M * tiles_n)) % gsz;
+    const int tn = (bid % (GROUP_M * tiles_n)) / gsz;
+    const int m0 = tm * BM, n0 = tn * BN;
+
+    const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
+    const int wm = wave % 4, wn = wave / 4;
+
+    // loader: instruction q of a tile moves 16 rows x 64 B (q < 16: A rows, else B rows);
+    // lane -> row lane/4, LDS chunk lane%4 holding global chunk (lane%4) ^ ((row>>2)&3)
+    const int lrow = lane / 4, lchunk = (lane & 3) ^ ((lane >> 4) & 3);
+    const half_t *gp[LPT];
+#pragma unroll
+    for (int t = 0; t < LPT; ++t) {
+        const int q = wave + t * NWAVES;
+        if (q < 16) {
+            int ar = m0 + q * 16 + lrow;
+            ar = ar < T ? ar : T - 1;
+            gp[t] = x + (size_t)ar * ldx + lchunk * 8;
+        } else {
+            int brl = (q - 16) * 16 + lrow;
+            const half_t *wb = w;
+            if (NB == 2 && brl >= BN) { wb = w2; brl -= BN; }
+            int br = n0 + brl;
+            br = br < N ? br : N - 1;
+            gp[t] = wb + (size_t)br * K + lchunk * 8;
+        }
+    }
+    auto issue = [&](int kt) {
+        half_t *st = lds + (kt % STAGES) * STAGE_HALVES;
+        const int k0 = kt * DMA_BK;
+#pragma unroll
+        for (int t = 0; t < LPT; ++t)
+            __builtin_amdgcn_global_load_lds(DMA_GP(gp[t] + k0), DMA_LP(st + (wave + t * NWAVES) * 16 * DMA_BK), 16, 0, 0);
+    };
+
+    const int frow = lane % 32, sw = (frow >> 2) & 3;
+    int a_off[2], b_off[2];
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+        const int pc = (ks * 2 + lane / 32) ^ sw;
+        a_off[ks] = (wm * 64 + frow) * DMA_BK + pc * 8;
+        b_off[ks] = BM * DMA_BK + ((NB == 1 ? wn * 128 : wn * 64) + frow) * DMA_BK + pc * 8;
+    }
+    half8_t af[2][FM], bf[2][4];
+    auto lfrag = [&](int set, int kt, int ks) {
+        const half_t *st = lds + (kt % STAGES) * STAGE_HALVES;
+#pragma unroll
+        for (int i = 0; i < FM; ++i) af[set][i] = load8(st + a_off[ks] + i * 32 * DMA_BK);
+#pragma unroll
+        for (int f = 0; f < 4; ++f) {
+            const int roff = NB == 1 ? f * 32 : (f / 2) * BN + (f % 2) * 32;
+            bf[set][f] = load8(st + b_off[ks] + roff * DMA_BK);
+        }
+    };
+
+    float16_t acc[4][FM];
+#pragma unroll
+    for (int f = 0; f < 4; ++f)
+#pragma unroll
+        for (int i = 0; i < FM; ++i)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[f][i][e] = 0.f;
+    auto mma = [&](int set) {
+#pragma unroll
+        for (int f = 0; f < 4; ++f)
+#pragma unroll
+            for (int i = 0; i < FM; ++i)
+                acc[f][i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[set][f], af[set][i], acc[f][i], 0, 0, 0);
+    };
+
+    const int nk = K / DMA_BK;
+#pragma unroll
+    for (int t = 0; t < AHEAD + (PREF ? 1 : 0); ++t)
+        if (t < nk) issue(t);
+    // tiles issued so far: min(nk, AHEAD + PREF).  Loop invariant at the top of iteration kt: tiles up to
+    // kt + (PREF ? 1 : 0) have landed for every wave, tiles up to kt + AHEAD - (PREF ? 0 : 1) ... are in flight.
+    if (PREF) {
+        const int beyond = (nk < AHEAD + 1 ? nk : AHEAD + 1) - 2;
+        if (beyond >= 2) dma_wait_barrier<2 * LPT>();
+        else if (beyond == 1) dma_wait_barrier<LPT>();
+        else dma_wait_barrier<0>();
+        lfrag(0, 0, 0);
+        for (int kt = 0; kt < nk; ++kt) {
+            __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0): fragments prefetched last iteration are in
+            if (kt + AHEAD + 1 < nk) issue(kt + AHEAD + 1);
+            lfrag(1, kt, 1);
+            __builtin_amdgcn_sched_barrier(0);
+            mma(0);
+            __builtin_amdgcn_sched_barrier(0);
+            if (kt + 1 < nk) lfrag(0, kt + 1, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            mma(1);
+            __builtin_amdgcn_sched_barrier(0);
+            const int last = kt + AHEAD + 1 < nk - 1 ? kt + AHEAD + 1 : nk - 1;
+            const int beyond2 = last - (kt + 2);
+            if (AHEAD >= 3 && beyond2 >= 2) dma_wait_barrier<2 * LPT>();
+            else if (beyond2 >= 1) dma_wait_barrier<LPT>();
+            else dma_wait_barrier<0>();
+        }
+    } else {
+        for (int kt = 0; kt < nk; ++kt) {
+            // tile kt landed?  loads issued after it: tiles kt+1 .. min(kt+AHEAD-1, nk-1)
+            const int last = kt + AHEAD - 1 < nk - 1 ? kt + AHEAD - 1 : nk - 1;
+            const int beyond = last - kt;
+            if (AHEAD >= 3 && beyond >= 2) dma_wait_barrier<2 * LPT>();
+            else if (beyond >= 1) dma_wait_barrier<LPT>();
+            else dma_wait_barrier<0>();
+            if (kt + AHEAD < nk) issue(kt + AHEAD);
+            lfrag(0, kt, 0);
+            lfrag(1, kt, 1);
+            __builtin_amdgcn_sched_barrier(0);
+            mma(0);
+            mma(1);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+
+    const int mrow = lane % 32, ncol0 = 4 * (lane / 32);
+#pragma unroll
+    for (int i = 0; i < FM; ++i) {
+        const int m = m0 + wm * 64 + i * 32 + mrow;
+        const int mc = m < T ? m : T - 1;
+#pragma unroll
+        for (int j = 0; j < FN; ++j) {
+            const int nb = n0 + (NB == 1 ? wn * 128 : wn * 64) + j * 32 + ncol0;
+            half4_t rv[4];
+            if (NB == 1 && res) {
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    int n = nb + 8 * g;
+                    n = n < N ? n : N - 4;
+                    rv[g] = *reinterpret_cast<const half4_t *>(res + (size_t)mc * ldr + n);
+                }
+            }
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int n = nb + 8 * g;
+                half4_t o;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    if (NB == 2) o[e] = (half_t)(silu_g(acc[j][i][4 * g + e]) * acc[2 + j][i][4 * g + e]);
+                    else if (res) o[e] = (half_t)((float)(half_t)acc[j][i][4 * g + e] + (float)rv[g][e]);
+                    else o[e] = (half_t)acc[j][i][4 * g + e];
+                }
+                if (m < T && n < N) *reinterpret_cast<half4_t *>(out + (size_t)m * ldo + n) = o;
+            }
+        }
+    }
+}
+
+template <int NB, int WGN, int STAGES, bool PREF, int OCC>
+static int gemm_dma_launch(const half_t *x, int ldx, const half_t *w, const half_t *w2, const half_t *res, int ldr,
+                        half_t *out, int ldo, int T, int N, int K, hipStream_t s) {
+    constexpr int BN = WGN * 128 / NB;
+    const int tiles_m = (T + 255) / 256, tiles_n = (N + BN - 1) / BN;
+    const size_t smem = sizeof(half_t) * (size_t)STAGES * (256 + WGN * 128) * DMA_BK;
+    auto kern = gemm_dma_kernel<NB, WGN, STAGES, PREF, OCC>;
+    static bool attr_set = false;
+    if (!attr_set) {
+        LLM_HIP_CHECK(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+        attr_set = true;
+    }
+    kern<<<dim3(tiles_m * tiles_n), dim3(WGN * 256), smem, s>>>(x, ldx, w, w2, res, ldr, out, ldo, T, N, K, tiles_m, tiles_n);
+    LLM_LAUNCH_CHECK("gemm_dma_kernel");
+    return LLM_OK;
+}
+
+// ---------------------------------------------------------------------------
 static int check_linear(const void *x, int ldx, const void *w, const void *out, int ldo, int T, int N, int K,
                         const char *who) {
     LLM_REQUIRE(x && w && out, "%s: null pointer", who);
@@ -310,6 +524,11 @@ static int check_linear(const void *x, int ldx, const void *w, const void *out, 
     LLM_REQUIRE(ldx >= K && ldx % 8 == 0 && ldo >= N, "%s: ldx=%d ldo=%d", who, ldx, ldo);
     LLM_REQUIRE(aligned16(x) && aligned16(w), "%s: x and w must be 16-byte aligned", who);
     return LLM_OK;
+}
+
+// the direct-to-LDS kernels store (and read the residual) four halves at a time
+static bool dma_ok(const half_t *out, int ldo, const half_t *res, int ldr) {
+    return ((uintptr_t)out & 7u) == 0 && ldo % 4 == 0 && (!res || (((uintptr_t)res & 7u) == 0 && ldr % 4 == 0));
 }
 
 extern "C" {
@@ -332,7 +551,13 @@ int llm_linear(const uint16_t *x, int ldx, const uint16_t *w, const uint16_t *re
     }
     if (T <= 64 || N < 256) return gemm_launch<64, 64, 2, 2, 1>(xp, ldx, wp, nullptr, rp, ldr, op, ldo, T, N, K, s);
     if (T <= 128) return gemm_launch<128, 128, 2, 2, 1>(xp, ldx, wp, nullptr, rp, ldr, op, ldo, T, N, K, s);
-    return gemm_launch<256, 256, 4, 2, 1>(xp, ldx, wp, nullptr, rp, ldr, op, ldo, T, N, K, s);
+    if (!dma_ok(op, ldo, rp, ldr)) return gemm_launch<128, 128, 2, 2, 1>(xp, ldx, wp, nullptr, rp, ldr, op, ldo, T, N, K, s);
+    // few tiles, short K: two independent 4-wave workgroups per CU hide each other's prologue and
+    // epilogue; otherwise the 8-wave 256 x 256 tile with the deeper pipeline wins
+    const long tiles = (long)((T + 255) / 256) * ((N + 255) / 256);
+    if (T <= 1024 || (tiles <= 512 && K <= 4096))
+        return gemm_dma_launch<1, 1, 3, false, 2>(xp, ldx, wp, nullptr, rp, ldr, op, ldo, T, N, K, s);
+    return gemm_dma_launch<1, 2, 4, true, 1>(xp, ldx, wp, nullptr, rp, ldr, op, ldo, T, N, K, s);
 }
 
 int llm_linear_swiglu(const uint16_t *x, int ldx, const uint16_t *wgate, const uint16_t *wup, uint16_t *out,
@@ -353,7 +578,9 @@ int llm_linear_swiglu(const uint16_t *x, int ldx, const uint16_t *wgate, const u
     }
     if (T <= 64 || N < 256) return gemm_launch<64, 64, 2, 2, 2>(xp, ldx, gp, up, nullptr, 0, op, ldo, T, N, K, s);
     if (T <= 128) return gemm_launch<128, 64, 2, 2, 2>(xp, ldx, gp, up, nullptr, 0, op, ldo, T, N, K, s);
-    return gemm_launch<256, 128, 4, 2, 2>(xp, ldx, gp, up, nullptr, 0, op, ldo, T, N, K, s);
+    if (!dma_ok(op, ldo, nullptr, 0)) return gemm_launch<128, 64, 2, 2, 2>(xp, ldx, gp, up, nullptr, 0, op, ldo, T, N, K, s);
+    if (T <= 1024) return gemm_dma_launch<2, 1, 3, false, 2>(xp, ldx, gp, up, nullptr, 0, op, ldo, T, N, K, s);
+    return gemm_dma_launch<2, 2, 4, true, 1>(xp, ldx, gp, up, nullptr, 0, op, ldo, T, N, K, s);
 }
 
 int llm_norm_linear(const uint16_t *x, const uint16_t *gain, double eps, const uint16_t *w, uint16_t *out, int N, int K,
