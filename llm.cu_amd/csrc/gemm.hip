@@ -318,23 +318,25 @@ template <int N> __device__ __forceinline__ void dma_wait_barrier() {
     asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(N) : "memory");
 }
 
-// 256 x (WGN*128) macro-tile, WGN*4 wavefronts each owning 64 x 128 of it (NB = 2: 64 columns of gate and
-// the same 64 of up), BK = 32, STAGES LDS buffers filled by direct global->LDS loads.
+// (WGM*64) x (WGN*128) macro-tile, WGM*WGN wavefronts each owning 64 x 128 of it (NB = 2: 64 columns of
+// gate and the same 64 of up), BK = 32, STAGES LDS buffers filled by direct global->LDS loads.
+// Split-K (ws != nullptr): workgroup (tile, z) covers k in [z*kper, (z+1)*kper) and stores its fp32
+// partial tile to ws[z][T][N]; splitk_reduce_kernel sums the slices in ascending z and finishes.
 // PREF: read the next tile's first fragments before the barrier (needs tiles kt and kt+1 landed at
 // barrier kt, so loads run STAGES-2 iterations ahead); otherwise loads run STAGES-1 ahead.
-template <int NB, int WGN, int STAGES, bool PREF, int OCC>
-__global__ __launch_bounds__(WGN * 256, OCC) void gemm_dma_kernel(const half_t *__restrict__ x, int ldx,
+template <int NB, int WGM, int WGN, int STAGES, bool PREF, int OCC>
+__global__ __launch_bounds__(WGM * WGN * 64, OCC) void gemm_dma_kernel(const half_t *__restrict__ x, int ldx,
                                                                const half_t *__restrict__ w, const half_t *__restrict__ w2,
                                                                const half_t *res, int ldr, half_t *out, int ldo, int T, int N, int K,
-                                                               int tiles_m, int tiles_n) {
-    constexpr int NWAVES = 4 * WGN;
-    constexpr int BM = 256, BROWS = WGN * 128; // B rows in a stage (both matrices when NB = 2)
+                                                               int tiles_m, int tiles_n, float *ws, int kper) {
+    constexpr int NWAVES = WGM * WGN;
+    constexpr int BM = WGM * 64, BROWS = WGN * 128; // B rows in a stage (both matrices when NB = 2)
     constexpr int BN = BROWS / NB;             // output columns per tile
     constexpr int FM = 2, FN = 4 / NB;
     constexpr int STAGE_HALVES = (BM + BROWS) * DMA_BK;
     constexpr int LPT = (BM + BROWS) / 16 / NWAVES; // load instructions per wave per tile
     constexpr int AHEAD = PREF ? STAGES - 2 : STAGES - 1;
-    static_assert(16 % NWAVES == 0 || NWAVES == 8, "loader split");
+    static_assert((BM + BROWS) / 16 % NWAVES == 0, "loader split");
     extern __shared__ __attribute__((aligned(16))) half_t lds[];
 
     const int nblk = tiles_m * tiles_n;
@@ -352,26 +354,27 @@ __global__ __launch_bounds__(WGN * 256, OCC) void gemm_dma_kernel(const half_t *
     const int m0 = tm * BM, n0 = tn * BN;
 
     const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
-    const int wm = wave % 4, wn = wave / 4;
+    const int wm = wave % WGM, wn = wave / WGM;
+    const int kbeg = ws ? blockIdx.y * kper : 0;
 
-    // loader: instruction q of a tile moves 16 rows x 64 B (q < 16: A rows, else B rows);
+    // loader: instruction q of a tile moves 16 rows x 64 B (q < BM/16: A rows, else B rows);
     // lane -> row lane/4, LDS chunk lane%4 holding global chunk (lane%4) ^ ((row>>2)&3)
     const int lrow = lane / 4, lchunk = (lane & 3) ^ ((lane >> 4) & 3);
     const half_t *gp[LPT];
 #pragma unroll
     for (int t = 0; t < LPT; ++t) {
         const int q = wave + t * NWAVES;
-        if (q < 16) {
+        if (q < BM / 16) {
             int ar = m0 + q * 16 + lrow;
             ar = ar < T ? ar : T - 1;
-            gp[t] = x + (size_t)ar * ldx + lchunk * 8;
+            gp[t] = x + (size_t)ar * ldx + kbeg + lchunk * 8;
         } else {
-            int brl = (q - 16) * 16 + lrow;
+            int brl = (q - BM / 16) * 16 + lrow;
             const half_t *wb = w;
             if (NB == 2 && brl >= BN) { wb = w2; brl -= BN; }
             int br = n0 + brl;
             br = br < N ? br : N - 1;
-            gp[t] = wb + (size_t)br * K + lchunk * 8;
+            gp[t] = wb + (size_t)br * K + kbeg + lchunk * 8;
         }
     }
     auto issue = [&](int kt) {
@@ -417,7 +420,7 @@ __global__ __launch_bounds__(WGN * 256, OCC) void gemm_dma_kernel(const half_t *
                 acc[f][i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[set][f], af[set][i], acc[f][i], 0, 0, 0);
     };
 
-    const int nk = K / DMA_BK;
+    const int nk = (ws ? kper : K) / DMA_BK;
 #pragma unroll
     for (int t = 0; t < AHEAD + (PREF ? 1 : 0); ++t)
         if (t < nk) issue(t);
@@ -465,6 +468,24 @@ __global__ __launch_bounds__(WGN * 256, OCC) void gemm_dma_kernel(const half_t *
     }
 
     const int mrow = lane % 32, ncol0 = 4 * (lane / 32);
+    if (NB == 1 && ws) {
+        float *wz = ws + (size_t)blockIdx.y * T * N;
+#pragma unroll
+        for (int i = 0; i < FM; ++i) {
+            const int m = m0 + wm * 64 + i * 32 + mrow;
+#pragma unroll
+            for (int j = 0; j < FN; ++j)
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const int n = n0 + wn * 128 + j * 32 + ncol0 + 8 * g;
+                    float4_t o;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) o[e] = acc[j][i][4 * g + e];
+                    if (m < T && n < N) *reinterpret_cast<float4_t *>(wz + (size_t)m * N + n) = o;
+                }
+        }
+        return;
+    }
 #pragma unroll
     for (int i = 0; i < FM; ++i) {
         const int m = m0 + wm * 64 + i * 32 + mrow;
@@ -497,21 +518,70 @@ __global__ __launch_bounds__(WGN * 256, OCC) void gemm_dma_kernel(const half_t *
     }
 }
 
-template <int NB, int WGN, int STAGES, bool PREF, int OCC>
+// out[m][n] = finish(sum over z of ws[z][m][n]): four columns per thread, slices added in ascending z
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const float *__restrict__ ws, int S, int T, int N,
+                                                            const half_t *res, int ldr, half_t *out, int ldo) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; // index of a group of four columns
+    const int n4 = N / 4;
+    if (i >= (size_t)T * n4) return;
+    const int m = (int)(i / n4), n = (int)(i % n4) * 4;
+    float4_t a = *reinterpret_cast<const float4_t *>(ws + (size_t)m * N + n);
+    for (int z = 1; z < S; ++z) {
+        const float4_t b = *reinterpret_cast<const float4_t *>(ws + ((size_t)z * T + m) * N + n);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) a[e] += b[e];
+    }
+    half4_t r = {0, 0, 0, 0}, o;
+    if (res) r = *reinterpret_cast<const half4_t *>(res + (size_t)m * ldr + n);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) o[e] = res ? (half_t)((float)(half_t)a[e] + (float)r[e]) : (half_t)a[e];
+    *reinterpret_cast<half4_t *>(out + (size_t)m * ldo + n) = o;
+}
+
+// fp32 partial tiles of split-K launches; one buffer per process, allocated by llm_init
+static float *g_splitk_ws = nullptr;
+static const size_t SPLITK_WS_BYTES = (size_t)64 << 20;
+
+int gemm_init_workspace() {
+    if (!g_splitk_ws) LLM_HIP_CHECK(hipMalloc((void **)&g_splitk_ws, SPLITK_WS_BYTES));
+    return LLM_OK;
+}
+
+template <int NB, int WGM, int WGN, int STAGES, bool PREF, int OCC>
 static int gemm_dma_launch(const half_t *x, int ldx, const half_t *w, const half_t *w2, const half_t *res, int ldr,
-                        half_t *out, int ldo, int T, int N, int K, hipStream_t s) {
-    constexpr int BN = WGN * 128 / NB;
-    const int tiles_m = (T + 255) / 256, tiles_n = (N + BN - 1) / BN;
-    const size_t smem = sizeof(half_t) * (size_t)STAGES * (256 + WGN * 128) * DMA_BK;
-    auto kern = gemm_dma_kernel<NB, WGN, STAGES, PREF, OCC>;
+                           half_t *out, int ldo, int T, int N, int K, int splits, hipStream_t s) {
+    constexpr int BM = WGM * 64, BN = WGN * 128 / NB;
+    const int tiles_m = (T + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
+    const size_t smem = sizeof(half_t) * (size_t)STAGES * (BM + WGN * 128) * DMA_BK;
+    auto kern = gemm_dma_kernel<NB, WGM, WGN, STAGES, PREF, OCC>;
     static bool attr_set = false;
     if (!attr_set) {
         LLM_HIP_CHECK(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
         attr_set = true;
     }
-    kern<<<dim3(tiles_m * tiles_n), dim3(WGN * 256), smem, s>>>(x, ldx, w, w2, res, ldr, out, ldo, T, N, K, tiles_m, tiles_n);
+    if (NB == 1 && splits > 1) {
+        kern<<<dim3(tiles_m * tiles_n, splits), dim3(WGM * WGN * 64), smem, s>>>(x, ldx, w, w2, nullptr, 0, out, ldo, T, N, K,
+                                                                               tiles_m, tiles_n, g_splitk_ws, K / splits);
+        LLM_LAUNCH_CHECK("gemm_dma_kernel (split-K)");
+        const size_t groups = (size_t)T * (N / 4);
+        splitk_reduce_kernel<<<dim3((unsigned)((groups + 255) / 256)), dim3(256), 0, s>>>(g_splitk_ws, splits, T, N, res, ldr, out, ldo);
+        LLM_LAUNCH_CHECK("splitk_reduce_kernel");
+        return LLM_OK;
+    }
+    kern<<<dim3(tiles_m * tiles_n), dim3(WGM * WGN * 64), smem, s>>>(x, ldx, w, w2, res, ldr, out, ldo, T, N, K, tiles_m,
+                                                                      tiles_n, nullptr, 0);
     LLM_LAUNCH_CHECK("gemm_dma_kernel");
     return LLM_OK;
+}
+
+// Number of k-slices for a launch with `tiles` output tiles: enough workgroups to put two on every CU,
+// slices of at least 256 k that divide K into multiples of DMA_BK, partial tiles that fit the workspace.
+static int pick_splits(long tiles, int T, int N, int K) {
+    int s = 1;
+    while (s < 8 && tiles * s < 256 && K % (2 * s * DMA_BK) == 0 && K / (2 * s) >= 256 &&
+           (size_t)(2 * s) * T * N * sizeof(float) <= SPLITK_WS_BYTES && g_splitk_ws)
+        s *= 2;
+    return s;
 }
 
 // ---------------------------------------------------------------------------
@@ -549,15 +619,25 @@ int llm_linear(const uint16_t *x, int ldx, const uint16_t *w, const uint16_t *re
         LLM_LAUNCH_CHECK("skinny_kernel");
         return LLM_OK;
     }
-    if (T <= 64 || N < 256) return gemm_launch<64, 64, 2, 2, 1>(xp, ldx, wp, nullptr, rp, ldr, op, ldo, T, N, K, s);
-    if (T <= 128) return gemm_launch<128, 128, 2, 2, 1>(xp, ldx, wp, nullptr, rp, ldr, op, ldo, T, N, K, s);
-    if (!dma_ok(op, ldo, rp, ldr)) return gemm_launch<128, 128, 2, 2, 1>(xp, ldx, wp, nullptr, rp, ldr, op, ldo, T, N, K, s);
+    if (!dma_ok(op, ldo, rp, ldr) || N < 128) {
+        if (T <= 64 || N < 256) return gemm_launch<64, 64, 2, 2, 1>(xp, ldx, wp, nullptr, rp, ldr, op, ldo, T, N, K, s);
+        return gemm_launch<128, 128, 2, 2, 1>(xp, ldx, wp, nullptr, rp, ldr, op, ldo, T, N, K, s);
+    }
+    if (T <= 128) {
+        // weight-streaming regime: 128 x 128 tiles, k split so that every CU has work
+        const long tiles = (long)((N + 127) / 128);
+        return gemm_dma_launch<1, 2, 1, 4, false, 2>(xp, ldx, wp, nullptr, rp, ldr, op, ldo, T, N, K,
+                                                     pick_splits(tiles, T, N, K), s);
+    }
     // few tiles, short K: two independent 4-wave workgroups per CU hide each other's prologue and
     // epilogue; otherwise the 8-wave 256 x 256 tile with the deeper pipeline wins
     const long tiles = (long)((T + 255) / 256) * ((N + 255) / 256);
-    if (T <= 1024 || (tiles <= 512 && K <= 4096))
-        return gemm_dma_launch<1, 1, 3, false, 2>(xp, ldx, wp, nullptr, rp, ldr, op, ldo, T, N, K, s);
-    return gemm_dma_launch<1, 2, 4, true, 1>(xp, ldx, wp, nullptr, rp, ldr, op, ldo, T, N, K, s);
+    if (T <= 1024 || (tiles <= 512 && K <= 4096)) {
+        const long t4 = (long)((T + 255) / 256) * ((N + 127) / 128);
+        return gemm_dma_launch<1, 4, 1, 3, false, 2>(xp, ldx, wp, nullptr, rp, ldr, op, ldo, T, N, K,
+                                                     pick_splits(t4, T, N, K), s);
+    }
+    return gemm_dma_launch<1, 4, 2, 4, true, 1>(xp, ldx, wp, nullptr, rp, ldr, op, ldo, T, N, K, 1, s);
 }
 
 int llm_linear_swiglu(const uint16_t *x, int ldx, const uint16_t *wgate, const uint16_t *wup, uint16_t *out,
@@ -576,11 +656,13 @@ int llm_linear_swiglu(const uint16_t *x, int ldx, const uint16_t *wgate, const u
         LLM_LAUNCH_CHECK("skinny_kernel<swiglu>");
         return LLM_OK;
     }
-    if (T <= 64 || N < 256) return gemm_launch<64, 64, 2, 2, 2>(xp, ldx, gp, up, nullptr, 0, op, ldo, T, N, K, s);
-    if (T <= 128) return gemm_launch<128, 64, 2, 2, 2>(xp, ldx, gp, up, nullptr, 0, op, ldo, T, N, K, s);
-    if (!dma_ok(op, ldo, nullptr, 0)) return gemm_launch<128, 64, 2, 2, 2>(xp, ldx, gp, up, nullptr, 0, op, ldo, T, N, K, s);
-    if (T <= 1024) return gemm_dma_launch<2, 1, 3, false, 2>(xp, ldx, gp, up, nullptr, 0, op, ldo, T, N, K, s);
-    return gemm_dma_launch<2, 2, 4, true, 1>(xp, ldx, gp, up, nullptr, 0, op, ldo, T, N, K, s);
+    if (!dma_ok(op, ldo, nullptr, 0) || N < 64) {
+        if (T <= 64 || N < 256) return gemm_launch<64, 64, 2, 2, 2>(xp, ldx, gp, up, nullptr, 0, op, ldo, T, N, K, s);
+        return gemm_launch<128, 64, 2, 2, 2>(xp, ldx, gp, up, nullptr, 0, op, ldo, T, N, K, s);
+    }
+    if (T <= 128) return gemm_dma_launch<2, 2, 1, 4, false, 2>(xp, ldx, gp, up, nullptr, 0, op, ldo, T, N, K, 1, s);
+    if (T <= 1024) return gemm_dma_launch<2, 4, 1, 3, false, 2>(xp, ldx, gp, up, nullptr, 0, op, ldo, T, N, K, 1, s);
+    return gemm_dma_launch<2, 4, 2, 4, true, 1>(xp, ldx, gp, up, nullptr, 0, op, ldo, T, N, K, 1, s);
 }
 
 int llm_norm_linear(const uint16_t *x, const uint16_t *gain, double eps, const uint16_t *w, uint16_t *out, int N, int K,

@@ -21,6 +21,8 @@ __global__ void fill_zero_kernel(uint32_t *p, size_t n_words) {
     for (; i < n_words; i += stride) p[i] = 0u;
 }
 
+int gemm_init_workspace(); // gemm.hip: split-K partial-sum buffer
+
 extern "C" {
 
 const char *llm_last_error(void) { return g_err; }
@@ -51,7 +53,7 @@ int llm_init(int device) {
         llm_set_error("device %d is %s; this library holds gfx950 code only", device, prop.gcnArchName);
         return LLM_ERR_NO_DEVICE;
     }
-    return LLM_OK;
+    return gemm_init_workspace();
 }
 
 int llm_device_name(char *buf, size_t n) {
