@@ -468,20 +468,22 @@ __global__ __launch_bounds__(WGM * WGN * 64, OCC) void gemm_dma_kernel(const hal
     }
 
     const int mrow = lane % 32, ncol0 = 4 * (lane / 32);
-    if (NB == 1 && ws) {
-        float *wz = ws + (size_t)blockIdx.y * T * N;
+    if (ws) {
+        // slice z holds NB planes of [T][N] fp32: the plain product, or gate then up
+        float *wz = ws + (size_t)blockIdx.y * NB * T * N;
 #pragma unroll
         for (int i = 0; i < FM; ++i) {
             const int m = m0 + wm * 64 + i * 32 + mrow;
 #pragma unroll
-            for (int j = 0; j < FN; ++j)
+            for (int f = 0; f < 4; ++f)
 #pragma unroll
                 for (int g = 0; g < 4; ++g) {
-                    const int n = n0 + wn * 128 + j * 32 + ncol0 + 8 * g;
+                    const int j = NB == 1 ? f : f % 2, plane = NB == 1 ? 0 : f / 2;
+                    const int n = n0 + (NB == 1 ? wn * 128 : wn * 64) + j * 32 + ncol0 + 8 * g;
                     float4_t o;
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) o[e] = acc[j][i][4 * g + e];
-                    if (m < T && n < N) *reinterpret_cast<float4_t *>(wz + (size_t)m * N + n) = o;
+                    for (int e = 0; e < 4; ++e) o[e] = acc[f][i][4 * g + e];
+                    if (m < T && n < N) *reinterpret_cast<float4_t *>(wz + ((size_t)plane * T + m) * N + n) = o;
                 }
         }
         return;
@@ -518,23 +520,32 @@ __global__ __launch_bounds__(WGM * WGN * 64, OCC) void gemm_dma_kernel(const hal
     }
 }
 
-// out[m][n] = finish(sum over z of ws[z][m][n]): four columns per thread, slices added in ascending z
+// out[m][n] = finish(sum over z of ws[z][m][n]) (NB = 2: SiLU(sum of gate slices) * sum of up slices):
+// four columns per thread, slices added in ascending z
+template <int NB>
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float *__restrict__ ws, int S, int T, int N,
                                                             const half_t *res, int ldr, half_t *out, int ldo) {
     const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; // index of a group of four columns
     const int n4 = N / 4;
     if (i >= (size_t)T * n4) return;
     const int m = (int)(i / n4), n = (int)(i % n4) * 4;
-    float4_t a = *reinterpret_cast<const float4_t *>(ws + (size_t)m * N + n);
-    for (int z = 1; z < S; ++z) {
-        const float4_t b = *reinterpret_cast<const float4_t *>(ws + ((size_t)z * T + m) * N + n);
+    float4_t a[NB];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) a[e] += b[e];
-    }
+    for (int b = 0; b < NB; ++b) a[b] = *reinterpret_cast<const float4_t *>(ws + ((size_t)b * T + m) * N + n);
+    for (int z = 1; z < S; ++z)
+#pragma unroll
+        for (int b = 0; b < NB; ++b) {
+            const float4_t v = *reinterpret_cast<const float4_t *>(ws + (((size_t)z * NB + b) * T + m) * N + n);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) a[b][e] += v[e];
+        }
     half4_t r = {0, 0, 0, 0}, o;
-    if (res) r = *reinterpret_cast<const half4_t *>(res + (size_t)m * ldr + n);
+    if (NB == 1 && res) r = *reinterpret_cast<const half4_t *>(res + (size_t)m * ldr + n);
 #pragma unroll
-    for (int e = 0; e < 4; ++e) o[e] = res ? (half_t)((float)(half_t)a[e] + (float)r[e]) : (half_t)a[e];
+    for (int e = 0; e < 4; ++e) {
+        if (NB == 2) o[e] = (half_t)(silu_g(a[0][e]) * a[NB - 1][e]);
+        else o[e] = res ? (half_t)((float)(half_t)a[0][e] + (float)r[e]) : (half_t)a[0][e];
+    }
     *reinterpret_cast<half4_t *>(out + (size_t)m * ldo + n) = o;
 }
 
@@ -559,12 +570,12 @@ static int gemm_dma_launch(const half_t *x, int ldx, const half_t *w, const half
         LLM_HIP_CHECK(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
         attr_set = true;
     }
-    if (NB == 1 && splits > 1) {
+    if (splits > 1) {
         kern<<<dim3(tiles_m * tiles_n, splits), dim3(WGM * WGN * 64), smem, s>>>(x, ldx, w, w2, nullptr, 0, out, ldo, T, N, K,
                                                                                tiles_m, tiles_n, g_splitk_ws, K / splits);
         LLM_LAUNCH_CHECK("gemm_dma_kernel (split-K)");
         const size_t groups = (size_t)T * (N / 4);
-        splitk_reduce_kernel<<<dim3((unsigned)((groups + 255) / 256)), dim3(256), 0, s>>>(g_splitk_ws, splits, T, N, res, ldr, out, ldo);
+        splitk_reduce_kernel<NB><<<dim3((unsigned)((groups + 255) / 256)), dim3(256), 0, s>>>(g_splitk_ws, splits, T, N, res, ldr, out, ldo);
         LLM_LAUNCH_CHECK("splitk_reduce_kernel");
         return LLM_OK;
     }
@@ -576,10 +587,10 @@ static int gemm_dma_launch(const half_t *x, int ldx, const half_t *w, const half
 
 // Number of k-slices for a launch with `tiles` output tiles: enough workgroups to put two on every CU,
 // slices of at least 256 k that divide K into multiples of DMA_BK, partial tiles that fit the workspace.
-static int pick_splits(long tiles, int T, int N, int K) {
+static int pick_splits(long tiles, int T, int N, int K, int planes = 1) {
     int s = 1;
     while (s < 8 && tiles * s < 256 && K % (2 * s * DMA_BK) == 0 && K / (2 * s) >= 256 &&
-           (size_t)(2 * s) * T * N * sizeof(float) <= SPLITK_WS_BYTES && g_splitk_ws)
+           (size_t)(2 * s) * planes * T * N * sizeof(float) <= SPLITK_WS_BYTES && g_splitk_ws)
         s *= 2;
     return s;
 }
@@ -660,7 +671,10 @@ int llm_linear_swiglu(const uint16_t *x, int ldx, const uint16_t *wgate, const u
         if (T <= 64 || N < 256) return gemm_launch<64, 64, 2, 2, 2>(xp, ldx, gp, up, nullptr, 0, op, ldo, T, N, K, s);
         return gemm_launch<128, 64, 2, 2, 2>(xp, ldx, gp, up, nullptr, 0, op, ldo, T, N, K, s);
     }
-    if (T <= 128) return gemm_dma_launch<2, 2, 1, 4, false, 2>(xp, ldx, gp, up, nullptr, 0, op, ldo, T, N, K, 1, s);
+    // (splitting k here costs more in fp32 partial traffic than the extra workgroups return)
+    if (T <= 128)
+        return gemm_dma_launch<2, 2, 1, 4, false, 2>(xp, ldx, gp, up, nullptr, 0, op, ldo, T, N, K,
+                                                     pick_splits((long)((N + 63) / 64), T, N, K, 2), s);
     if (T <= 1024) return gemm_dma_launch<2, 4, 1, 3, false, 2>(xp, ldx, gp, up, nullptr, 0, op, ldo, T, N, K, 1, s);
     return gemm_dma_launch<2, 4, 2, 4, true, 1>(xp, ldx, gp, up, nullptr, 0, op, ldo, T, N, K, 1, s);
 }
