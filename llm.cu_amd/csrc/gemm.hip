@@ -674,7 +674,7 @@ int llm_linear_swiglu(const uint16_t *x, int ldx, const uint16_t *wgate, const u
     // (splitting k here costs more in fp32 partial traffic than the extra workgroups return)
     if (T <= 128)
         return gemm_dma_launch<2, 2, 1, 4, false, 2>(xp, ldx, gp, up, nullptr, 0, op, ldo, T, N, K,
-                                                     pick_splits((long)((N + 63) / 64), T, N, K, 2), s);
+                                                     pick_splits(2 * (long)((N + 63) / 64), T, N, K, 2), s);
     if (T <= 1024) return gemm_dma_launch<2, 4, 1, 3, false, 2>(xp, ldx, gp, up, nullptr, 0, op, ldo, T, N, K, 1, s);
     return gemm_dma_launch<2, 4, 2, 4, true, 1>(xp, ldx, gp, up, nullptr, 0, op, ldo, T, N, K, 1, s);
 }
