@@ -81,6 +81,12 @@ typedef struct {
     void *engine; /* extension: opaque engine state (KV cache, scratch, stream, graph) */
 } CudaCache;
 
+/* src/inference/inference.cuh:46-49 */
+typedef struct {
+    float probability;
+    int index;
+} ProbIndex;
+
 /* ---- reference API ---------------------------------------------------- */
 Llama3 *init_llama3(int n_layers);
 void free_llama3(Llama3 *llama3);
@@ -92,7 +98,23 @@ int *tokens_to_cuda(int *tokens, int embed_size, Tensor *token_tensor);
 /* h_tokens[0] = n+1, ids in h_tokens[1..n]; returns the next token id. */
 int inference(Llama3 *llama3_model, Tensor *X, int *d_tokens, int *h_tokens, CudaCache *Cache);
 
+/* Host sampler, src/inference/inference.cuh:418-426, inference.cu:1030-1161: temperature 0.7, top-k 50
+ * (renormalises the head of the sorted array in place, its own draw is discarded), top-p 0.9 picks the
+ * token; rand() unseeded.  tensor: vocab floats of scratch, half_tensor: the fp16 logits. */
+int sample_next_token(float *tensor, llm_half *half_tensor);
+ProbIndex *temperature_softmax(float *tensor, llm_half *half_tensor, float temperature);
+int _compare_desc(const void *a, const void *b);
+int top_k_sampling(ProbIndex *prob_dist_array, int k);
+int top_p_sampling(ProbIndex *prob_dist_array, float p);
+
 /* ---- extensions -------------------------------------------------------- */
+/* The reference fixes vocab 128256, temperature 0.7, top-k 50, top-p 0.9 at compile time
+ * (inference.cu:24-29); init_cache_cfg() sets the vocabulary, this sets all four. */
+void llama3_sampler_config(int vocab, float temperature, int top_k, float top_p);
+/* inference() returns the greedy id (0, default) or sample_next_token() of the logits as the
+ * reference does (1). */
+void llama3_set_sampling(CudaCache *c, int on);
+
 typedef struct {
     int n_layers;
     int d_model;

@@ -154,6 +154,13 @@ HOST_ABI = {
     "seeded_fill_model": (None, [_LP, C.POINTER(ModelConfig), _u64]),
     "seeded_write_safetensors": (_i, [C.POINTER(ModelConfig), _u64, C.c_char_p]),
     "seeded_tensor_id": (_u64, [_i, _i]),
+    "sample_next_token": (_i, [_vp, _vp]),
+    "temperature_softmax": (_vp, [_vp, _vp, C.c_float]),
+    "_compare_desc": (_i, [_vp, _vp]),
+    "top_k_sampling": (_i, [_vp, _i]),
+    "top_p_sampling": (_i, [_vp, C.c_float]),
+    "llama3_sampler_config": (None, [_i, C.c_float, _i, C.c_float]),
+    "llama3_set_sampling": (None, [_CP, _i]),
 }
 
 _lib = None

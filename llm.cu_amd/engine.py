@@ -155,6 +155,10 @@ class Engine:
         arr[1:n + 1] = tokens
         return lib().inference(self.model.handle, None, None, arr.ctypes.data_as(C.POINTER(C.c_int)), self.cache)
 
+    def set_sampling(self, on):
+        """inference() returns the reference's temperature/top-k/top-p sample (True) or the argmax (False)."""
+        lib().llama3_set_sampling(self.cache, 1 if on else 0)
+
     def close(self):
         if self.cache:
             lib().free_cache(self.cache)

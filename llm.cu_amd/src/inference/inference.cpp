@@ -49,6 +49,7 @@ struct Engine {
     std::vector<int> tokens; // ids whose K/V are cached
     int pos = 0;
     bool use_graph = true;
+    bool sampling = false; // inference() samples like the reference instead of returning the argmax
     llm_graph_t graph = nullptr;
     llm_event_t ev[4] = {nullptr, nullptr, nullptr, nullptr};
 };
@@ -296,6 +297,7 @@ extern "C" CudaCache *init_cache_cfg(Llama3 *m, const ModelConfig *cfg) {
     C->d_token_probdist = e->logits;
     C->h_token_probdist = (llm_half *)malloc(sizeof(llm_half) * (size_t)c.vocab);
     C->f_token_probdist = (float *)malloc(sizeof(float) * (size_t)c.vocab);
+    llama3_sampler_config(c.vocab, 0.7f, 50, 0.9f); // inference.cu:27-29
     C->engine = e;
     return C;
 }
@@ -463,5 +465,8 @@ extern "C" int inference(Llama3 *m, Tensor *X, int *d_tokens, int *h_tokens, Cud
     const int fresh = n - e->pos;
     int tok = fresh == 1 ? llama3_decode(m, C, ids[n - 1]) : llama3_prefill(m, C, ids + e->pos, fresh);
     llama3_read_logits(C, C->h_token_probdist);
+    if (e->sampling) tok = sample_next_token(C->f_token_probdist, C->h_token_probdist); // inference.cu:1028
     return tok;
 }
+
+extern "C" void llama3_set_sampling(CudaCache *C, int on) { eng(C)->sampling = on != 0; }

@@ -725,3 +725,94 @@ int orc_model_forward_recompute(const orc_config *c, const orc_weights *w, const
     free(X); free(PN); free(Q); free(K); free(V); free(H); free(A);
     return tok;
 }
+
+/* ------------------------------------------------------------------ */
+/* Host sampler (inference.cu:1030-1161).                               */
+/* ------------------------------------------------------------------ */
+/* glibc random_r.c, TYPE_3 (degree 31, separation 3): srandom fills r[0..30] with the Lehmer sequence
+ * 16807*x mod (2^31-1) by Schrage's method, then discards 310 outputs. */
+void orc_rand_seed(orc_rand_state *s, unsigned seed) {
+    if (seed == 0) seed = 1;
+    s->r[0] = (int32_t)seed;
+    for (int i = 1; i < 31; ++i) {
+        long hi = s->r[i - 1] / 127773, lo = s->r[i - 1] % 127773;
+        long word = 16807 * lo - 2836 * hi;
+        if (word < 0) word += 2147483647;
+        s->r[i] = (int32_t)word;
+    }
+    s->f = 3;
+    s->b = 0;
+    for (int i = 0; i < 310; ++i) (void)orc_rand_next(s);
+}
+
+int orc_rand_next(orc_rand_state *s) {
+    uint32_t v = (uint32_t)s->r[s->f] + (uint32_t)s->r[s->b];
+    s->r[s->f] = (int32_t)v;
+    s->f = (s->f + 1) % 31;
+    s->b = (s->b + 1) % 31;
+    return (int)(v >> 1);
+}
+
+typedef struct { float probability; int index; } orc_prob; /* inference.cuh:46-49 */
+
+static int cmp_desc(const void *a, const void *b) { /* inference.cu:1074-1084 */
+    const orc_prob *x = (const orc_prob *)a, *y = (const orc_prob *)b;
+    if (x->probability < y->probability) return 1;
+    if (x->probability > y->probability) return -1;
+    return 0;
+}
+
+int orc_sample(const uint16_t *logits, int vocab, float temperature, int top_k, float top_p, orc_rand_state *s) {
+    const float rand_max = 2147483647.0f; /* (float)RAND_MAX */
+    orc_prob *arr = (orc_prob *)malloc((size_t)vocab * sizeof(orc_prob));
+    float *t = (float *)malloc((size_t)vocab * sizeof(float));
+    /* temperature_softmax, :1043-1072: no max subtraction, float running sum in index order */
+    float cumsum = 0.0f;
+    for (int i = 0; i < vocab; ++i) {
+        t[i] = expf(h2f(logits[i]) / temperature);
+        cumsum += t[i];
+    }
+    for (int i = 0; i < vocab; ++i) {
+        t[i] /= cumsum;
+        arr[i].probability = t[i];
+        arr[i].index = i;
+    }
+    qsort(arr, (size_t)vocab, sizeof(orc_prob), cmp_desc);
+    int tok;
+    /* top_k_sampling, :1086-1113: its return value is overwritten by the caller (:1034-1035) but the
+     * renormalised head of arr and the consumed draw remain */
+    if (top_k <= 0) {
+        (void)(orc_rand_next(s) % vocab);
+    } else {
+        int k = top_k > vocab ? vocab : top_k;
+        float sum = 0.0f;
+        for (int i = 0; i < k; ++i) sum += arr[i].probability;
+        for (int i = 0; i < k; ++i) arr[i].probability /= sum;
+        (void)orc_rand_next(s);
+    }
+    /* top_p_sampling, :1115-1161 */
+    if (top_p <= 0.0f) {
+        tok = arr[orc_rand_next(s) % vocab].index;
+    } else {
+        float p = top_p > 1.0f ? 1.0f : top_p;
+        float cumulative = 0.0f;
+        int cutoff = 0;
+        for (; cutoff < vocab; ++cutoff) {
+            cumulative += arr[cutoff].probability;
+            if (cumulative >= p) break;
+        }
+        const float sum = cumulative;
+        if (cutoff >= vocab) cutoff = vocab - 1;
+        for (int i = 0; i <= cutoff; ++i) arr[i].probability /= sum;
+        const float r = (float)orc_rand_next(s) / rand_max;
+        cumulative = 0.0f;
+        tok = arr[0].index;
+        for (int i = 0; i <= cutoff; ++i) {
+            cumulative += arr[i].probability;
+            if (r < cumulative) { tok = arr[i].index; break; }
+        }
+    }
+    free(arr);
+    free(t);
+    return tok;
+}

@@ -107,6 +107,17 @@ int orc_model_forward_recompute(const orc_config *cfg, const orc_weights *w,
 
 int orc_num_threads(void);
 
+/* ---- host sampler (inference.cu:1030-1161) ------------------------------ */
+/* glibc's rand() as the reference uses it (never seeded, i.e. srand(1)): the TYPE_3 additive-feedback
+ * generator r[i] = r[i-3] + r[i-31], output r[i] >> 1, restated so that the oracle keeps a private
+ * stream.  state: 34 + 2 words. */
+typedef struct { int32_t r[34]; int f, b; } orc_rand_state;
+void orc_rand_seed(orc_rand_state *s, unsigned seed);
+int  orc_rand_next(orc_rand_state *s); /* 0 .. 2^31-1 */
+/* One call of sample_next_token(): temperature softmax, qsort, top-k (draw discarded, renormalisation
+ * kept), top-p.  Consumes two draws when top_k > 0 and top_p > 0. */
+int orc_sample(const uint16_t *logits, int vocab, float temperature, int top_k, float top_p, orc_rand_state *s);
+
 #ifdef __cplusplus
 }
 #endif

@@ -102,6 +102,11 @@ def lib():
                                                   i32, vp, vp]
         L.orc_model_forward_recompute.restype = i32
         L.orc_num_threads.restype = i32
+        L.orc_rand_seed.argtypes = [vp, C.c_uint]
+        L.orc_rand_next.argtypes = [vp]
+        L.orc_rand_next.restype = i32
+        L.orc_sample.argtypes = [vp, i32, C.c_float, i32, C.c_float, vp]
+        L.orc_sample.restype = i32
         _lib = L
     return _lib
 
@@ -301,3 +306,19 @@ def forward_recompute(cfg, weights, tokens, want_hidden=False):
 
 def num_threads():
     return lib().orc_num_threads()
+
+
+class Rand:
+    """The oracle's private copy of glibc rand() (state seeded like srand(seed))."""
+
+    def __init__(self, seed=1):
+        self._s = (C.c_int32 * 36)()
+        lib().orc_rand_seed(self._s, seed)
+
+    def next(self):
+        return lib().orc_rand_next(self._s)
+
+
+def sample(logits, rng, temperature=0.7, top_k=50, top_p=0.9):
+    logits = _u16(logits)
+    return lib().orc_sample(_p(logits), logits.size, temperature, top_k, top_p, rng._s)

@@ -83,6 +83,17 @@ def test_reference_shaped_inference_call(gpu):
     eng.reset()
     t2, _ = eng.prefill(np.array(other, np.int32))
     assert t1 == t2
+    # the reference's own next-token rule: host sampler over the fp16 logits, libc rand() never seeded
+    libc = C.CDLL("libc.so.6")
+    eng.set_sampling(True)
+    libc.srand(1)
+    rnd = orc.Rand(1)
+    seq = list(prompt)
+    for _ in range(6):
+        tok = eng.inference(seq)
+        assert tok == orc.sample(eng.logits(), rnd)
+        seq.append(tok)
+    eng.set_sampling(False)
     eng.close()
     model.close()
 
