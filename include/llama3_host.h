@@ -102,6 +102,9 @@ int inference(Llama3 *llama3_model, Tensor *X, int *d_tokens, int *h_tokens, Cud
  * (renormalises the head of the sorted array in place, its own draw is discarded), top-p 0.9 picks the
  * token; rand() unseeded.  tensor: vocab floats of scratch, half_tensor: the fp16 logits. */
 int sample_next_token(float *tensor, llm_half *half_tensor);
+/* the same token through the reference's exact sequence of calls (full-vocabulary qsort per token);
+ * sample_next_token() reaches it by selecting only the top_k head when that is provably equivalent */
+int sample_next_token_reference(float *tensor, llm_half *half_tensor);
 ProbIndex *temperature_softmax(float *tensor, llm_half *half_tensor, float temperature);
 int _compare_desc(const void *a, const void *b);
 int top_k_sampling(ProbIndex *prob_dist_array, int k);

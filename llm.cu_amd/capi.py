@@ -155,6 +155,7 @@ HOST_ABI = {
     "seeded_write_safetensors": (_i, [C.POINTER(ModelConfig), _u64, C.c_char_p]),
     "seeded_tensor_id": (_u64, [_i, _i]),
     "sample_next_token": (_i, [_vp, _vp]),
+    "sample_next_token_reference": (_i, [_vp, _vp]),
     "temperature_softmax": (_vp, [_vp, _vp, C.c_float]),
     "_compare_desc": (_i, [_vp, _vp]),
     "top_k_sampling": (_i, [_vp, _i]),

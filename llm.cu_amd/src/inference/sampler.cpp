@@ -3,6 +3,7 @@
 // vocabulary, a top-k pass whose renormalisation of the first k entries stays in the array and whose
 // draw is thrown away, then the top-p pass that picks the token.  Randomness is the C library's rand(),
 // unseeded in the reference, so the stream is shared with every other caller in the process.
+#include <algorithm>
 #include <cmath>
 #include <cstdint>
 #include <cstdlib>
@@ -114,12 +115,62 @@ int top_p_sampling(ProbIndex *arr, float p) {
     return arr[0].index;
 }
 
-// inference.cu:1030-1041
-int sample_next_token(float *tensor, llm_half *half_tensor) {
+// inference.cu:1030-1041, call for call (a full qsort of the vocabulary per token: ~10 ms at 128256)
+int sample_next_token_reference(float *tensor, llm_half *half_tensor) {
     ProbIndex *arr = temperature_softmax(tensor, half_tensor, g_temperature);
     int selected = top_k_sampling(arr, g_top_k);
     selected = top_p_sampling(arr, g_top_p);
     free(arr);
+    return selected;
+}
+
+// Same result without sorting the vocabulary.  After top_k_sampling() has renormalised the first k
+// entries they sum to 1 up to rounding, so for top_p below that sum top_p_sampling() never looks past
+// entry k-1: only the k largest probabilities, in the order qsort leaves them, matter.  glibc's qsort
+// is a merge sort (stable) whenever it can allocate its buffer, so equal probabilities stay in index
+// order; partial_sort with the index as second key reproduces that head exactly.  Falls back to the
+// full path for settings where the tail of the array is reachable.
+int sample_next_token(float *tensor, llm_half *half_tensor) {
+    const int k = g_top_k;
+    if (k <= 0 || k >= g_vocab || !(g_top_p > 0.0f) || g_top_p > 0.99f)
+        return sample_next_token_reference(tensor, half_tensor);
+    float cumsum = 0.0f;
+    for (int i = 0; i < g_vocab; ++i) {
+        tensor[i] = expf(half_to_float(half_tensor[i]) / g_temperature);
+        cumsum += tensor[i];
+    }
+    for (int i = 0; i < g_vocab; ++i) tensor[i] /= cumsum;
+    // NaN probabilities (exp overflow) defeat every comparison: let the reference path decide
+    if (!(cumsum < INFINITY) || !(cumsum > 0.0f)) return sample_next_token_reference(tensor, half_tensor);
+    // k largest by (probability desc, index asc): threshold pass, then a sort of the few survivors
+    ProbIndex *head = (ProbIndex *)malloc((size_t)(2 * k + 64) * sizeof(ProbIndex));
+    if (!head) llama3_fail("sample_next_token: out of memory");
+    int n = 0;
+    const int cap = 2 * k + 64;
+    float floor_p = -1.0f; // entries below the current k-th best cannot enter the head
+    auto better = [](const ProbIndex &a, const ProbIndex &b) {
+        return a.probability > b.probability || (a.probability == b.probability && a.index < b.index);
+    };
+    for (int i = 0; i < g_vocab; ++i) {
+        const float p = tensor[i];
+        if (p < floor_p) continue; // ties with the floor come later in index order only if p == floor: keep them
+        head[n].probability = p;
+        head[n].index = i;
+        if (++n == cap) {
+            std::partial_sort(head, head + k, head + n, better);
+            n = k;
+            floor_p = head[k - 1].probability;
+        }
+    }
+    if (n > k) {
+        std::partial_sort(head, head + k, head + n, better);
+        n = k;
+    } else {
+        std::sort(head, head + n, better);
+    }
+    int selected = top_k_sampling(head, k);
+    selected = top_p_sampling(head, g_top_p);
+    free(head);
     return selected;
 }
 

@@ -158,3 +158,28 @@ def test_shipped_half_widening_all_patterns(pkg):
     assert np.allclose(scratch / scratch.max(), want / want.max(), rtol=1e-6, atol=0)
     assert abs(float(scratch.astype(np.float64).sum()) - 1.0) < 1e-4
     lib.llama3_sampler_config(128256, 0.7, 50, 0.9)
+
+
+def test_fast_head_selection_equals_the_full_sort_path(pkg):
+    """sample_next_token() selects only the top-k head; sample_next_token_reference() is the reference's
+    call sequence with the full qsort.  fp16 logits at vocabulary size tie constantly, so the order among
+    equal probabilities is exercised on every draw."""
+    import time
+    lib = pkg.lib()
+    libc = C.CDLL("libc.so.6")
+    rng = np.random.default_rng(5)
+    for vocab, n, scale in ((300, 200, 1.0), (4096, 100, 0.5), (128256, 6, 2.0), (128256, 3, 0.01)):
+        lib.llama3_sampler_config(vocab, 0.7, 50, 0.9)
+        scratch = np.empty(vocab, np.float32)
+        cases = [_logits(rng, vocab, scale) for _ in range(n)]
+        libc.srand(11)
+        t0 = time.time()
+        fast = [lib.sample_next_token(scratch.ctypes.data, lg.ctypes.data) for lg in cases]
+        t1 = time.time()
+        libc.srand(11)
+        full = [lib.sample_next_token_reference(scratch.ctypes.data, lg.ctypes.data) for lg in cases]
+        t2 = time.time()
+        assert fast == full
+        print("vocab %d: head selection %.3f ms per token, full sort %.3f ms" % (vocab, 1e3 * (t1 - t0) / n, 1e3 * (t2 - t1) / n))
+    lib.llama3_sampler_config(128256, 0.7, 50, 0.9)
+    libc.srand(1)
