@@ -165,6 +165,13 @@ int llm_attn_decode_rope(const uint16_t *qkv_dev, uint16_t *k_cache_dev, uint16_
                          uint16_t *out_dev, int pos_host, const int32_t *pos_dev, const float *table_dev,
                          int n_heads, int n_kv_heads, int head_dim, int max_pos, void *workspace_dev,
                          llm_stream_t stream);
+/* The same operation as two launches: one workgroup per (KV head, 256-position span) leaves partial
+ * softmax statistics and P.V, a second kernel (one workgroup per query head) merges them.  Correct at
+ * any position; faster than the single launch beyond 512 cached positions (no in-kernel merge tail). */
+int llm_attn_decode_rope_long(const uint16_t *qkv_dev, uint16_t *k_cache_dev, uint16_t *v_cache_dev,
+                         uint16_t *out_dev, int pos_host, const int32_t *pos_dev, const float *table_dev,
+                         int n_heads, int n_kv_heads, int head_dim, int max_pos, void *workspace_dev,
+                         llm_stream_t stream);
 /* Same attention for T query rows at positions pos0..pos0+T-1 (prompt pass),
  * streaming softmax on MFMA tiles; never materialises [H,T,T].
  * q: [T, ldq] with head h at columns h*hd; out: [T, ldo].  Cache rows beyond

@@ -45,7 +45,7 @@ struct AdArgs {
 // that write.
 //
 // NDIM is the number of head dims this workgroup produces, LS the span length.
-template <int HD, int G, bool FUSED, int NDIM, int LS>
+template <int HD, int G, bool FUSED, int NDIM, int LS, bool TWOPASS = false>
 __device__ __forceinline__ void attn_decode_body(const AdArgs &a, float *sc, half_t *qs, half_t *knew, half_t *vnew,
                                                  float *s_m, float *s_l, int *s_last, const int pos,
                                                  const int n_active, const int split, const int d_begin,
@@ -214,7 +214,7 @@ __device__ __forceinline__ void attn_decode_body(const AdArgs &a, float *sc, hal
             }
         }
         if (jc == 0) {
-            if (n_active == 1) {
+            if (n_active == 1 && !TWOPASS) {
 #pragma unroll
                 for (int h = 0; h < G; ++h) a.out[(size_t)(kvh * G + h) * HD + d] = (half_t)(acc[h] / s_l[h]);
             } else {
@@ -223,11 +223,13 @@ __device__ __forceinline__ void attn_decode_body(const AdArgs &a, float *sc, hal
             }
         }
     }
-    if (n_active == 1) return;
+    if (n_active == 1 && !TWOPASS) return;
     if (tid < G) {
         a.ws_ml[(((size_t)kvh * splits + split) * G + tid) * 2 + 0] = s_m[tid];
         a.ws_ml[(((size_t)kvh * splits + split) * G + tid) * 2 + 1] = s_l[tid];
     }
+
+    if (TWOPASS) return; // attn_merge_kernel combines the spans
 
     // ---- 6. the last workgroup of this head merges the spans ------------------------------------
     __threadfence();
@@ -339,6 +341,129 @@ static int dispatch_decode(AdArgs a, int n_heads, int head_dim, void *ws, hipStr
     return LLM_ERR_INVALID;
 }
 
+// ---------------------------------------------------------------------------
+// Long contexts: two launches.  attn_span_kernel gives every (KV head, 256-position span) its own
+// workgroup and leaves (max, sum, unnormalised P.V) per span; attn_merge_kernel, one workgroup per
+// query head, combines them.  No fence, counter or last-workgroup tail: beyond a few spans that tail
+// costs more than the second launch.
+// ---------------------------------------------------------------------------
+#define AD_LONG_LS 256
+#define AD_MERGE_THREADS 512
+
+template <int HD, int G, bool FUSED>
+__global__ __launch_bounds__(AD_THREADS) void attn_span_kernel(const AdArgs a) {
+    __shared__ float sc[G * AD_LONG_LS];
+    __shared__ __attribute__((aligned(16))) half_t qs[G * HD];
+    __shared__ __attribute__((aligned(16))) half_t knew[HD];
+    __shared__ __attribute__((aligned(16))) half_t vnew[HD];
+    __shared__ float s_m[G], s_l[G];
+    __shared__ int s_last;
+    int pos = a.pos_host + (a.pos_dev ? *a.pos_dev : 0);
+    if (pos > a.max_pos - 1) pos = a.max_pos - 1;
+    if (pos < 0) pos = 0;
+    const int n_active = pos / AD_LONG_LS + 1;
+    const int y = blockIdx.y;
+    if (y >= n_active) return;
+    attn_decode_body<HD, G, FUSED, HD, AD_LONG_LS, true>(a, sc, qs, knew, vnew, s_m, s_l, &s_last, pos, n_active, y, 0,
+                                                         y == n_active - 1);
+}
+
+template <int HD, int G>
+__global__ __launch_bounds__(AD_MERGE_THREADS) void attn_merge_kernel(const AdArgs a) {
+    constexpr int PARTS = AD_MERGE_THREADS / HD;
+    __shared__ float w[AD_MAX_SPLITS];
+    __shared__ float red[2 * AD_MERGE_THREADS / 64];
+    __shared__ float part_o[AD_MERGE_THREADS];
+    __shared__ float s_M, s_L;
+    int pos = a.pos_host + (a.pos_dev ? *a.pos_dev : 0);
+    if (pos > a.max_pos - 1) pos = a.max_pos - 1;
+    if (pos < 0) pos = 0;
+    const int n = pos / AD_LONG_LS + 1;
+    const int h = blockIdx.x, kvh = h / G, hh = h % G, splits = a.splits;
+    const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
+    float m = -FLT_MAX, l = 0.f;
+    if (tid < n) {
+        const size_t b = ((size_t)kvh * splits + tid) * G + hh;
+        m = a.ws_ml[b * 2];
+        l = a.ws_ml[b * 2 + 1];
+    }
+    float mx = wave_max(m);
+    if (lane == 0) red[wave] = mx;
+    __syncthreads();
+    if (tid == 0) {
+        float t = red[0];
+        for (int q = 1; q < AD_MERGE_THREADS / 64; ++q) t = fmaxf(t, red[q]);
+        s_M = t;
+    }
+    __syncthreads();
+    const float wgt = tid < n ? expf(m - s_M) : 0.f;
+    if (tid < n) w[tid] = wgt;
+    float ls = wave_sum(l * wgt);
+    if (lane == 0) red[AD_MERGE_THREADS / 64 + wave] = ls;
+    __syncthreads();
+    if (tid == 0) {
+        float t = 0.f;
+        for (int q = 0; q < AD_MERGE_THREADS / 64; ++q) t += red[AD_MERGE_THREADS / 64 + q];
+        s_L = t;
+    }
+    const int d = tid % HD, part = tid / HD;
+    // four spans per round: their loads are independent, so a round costs one trip to memory
+    float o = 0.f;
+    const float *accp = a.ws_acc + ((size_t)kvh * splits * G + hh) * HD + d;
+    int s = part;
+    for (; s + 3 * PARTS < n; s += 4 * PARTS) {
+        float v[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) v[u] = accp[(size_t)(s + u * PARTS) * G * HD];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) o += v[u] * w[s + u * PARTS];
+    }
+    for (; s < n; s += PARTS) o += accp[(size_t)s * G * HD] * w[s];
+    part_o[tid] = o;
+    __syncthreads();
+    if (tid < HD) {
+        float t = part_o[tid];
+#pragma unroll
+        for (int q = 1; q < PARTS; ++q) t += part_o[tid + q * HD];
+        a.out[(size_t)h * HD + tid] = (half_t)(t / s_L);
+    }
+}
+
+template <int HD, int G, bool FUSED>
+static int launch_decode_long(AdArgs a, void *ws, hipStream_t s) {
+    const int Hq = a.n_kv_heads * G;
+    a.ws_acc = (float *)ws;
+    a.ws_ml = a.ws_acc + (size_t)Hq * AD_MAX_SPLITS * HD;
+    a.counters = nullptr;
+    const int splits = (a.max_pos + AD_LONG_LS - 1) / AD_LONG_LS;
+    LLM_REQUIRE(splits <= AD_MAX_SPLITS, "llm_attn_decode: max_pos=%d exceeds %d", a.max_pos, AD_MAX_SPLITS * AD_LONG_LS);
+    a.splits = splits;
+    // with the position known on the host only the spans in use are launched
+    const int gy = a.pos_dev ? splits : a.pos_host / AD_LONG_LS + 1;
+    attn_span_kernel<HD, G, FUSED><<<dim3(a.n_kv_heads, gy), dim3(AD_THREADS), 0, s>>>(a);
+    LLM_LAUNCH_CHECK("attn_span_kernel");
+    attn_merge_kernel<HD, G><<<dim3(Hq), dim3(AD_MERGE_THREADS), 0, s>>>(a);
+    LLM_LAUNCH_CHECK("attn_merge_kernel");
+    return LLM_OK;
+}
+
+template <bool FUSED>
+static int dispatch_decode_long(AdArgs a, int n_heads, int head_dim, void *ws, hipStream_t s) {
+    const int G = n_heads / a.n_kv_heads;
+#define AD_CASE(HD_, G_) \
+    if (head_dim == HD_ && G == G_) return launch_decode_long<HD_, G_, FUSED>(a, ws, s);
+    AD_CASE(128, 4)
+    AD_CASE(128, 8)
+    AD_CASE(128, 1)
+    AD_CASE(64, 4)
+    AD_CASE(64, 1)
+    AD_CASE(32, 4)
+    AD_CASE(32, 1)
+#undef AD_CASE
+    llm_set_error("llm_attn_decode: head_dim=%d with group size %d is not built", head_dim, G);
+    return LLM_ERR_INVALID;
+}
+
 extern "C" {
 
 // Layout: acc [Hq][AD_MAX_SPLITS][hd] floats, (m,l) [Hq][AD_MAX_SPLITS][2]
@@ -389,6 +514,28 @@ int llm_attn_decode_rope(const uint16_t *qkv, uint16_t *kc, uint16_t *vc, uint16
     a.n_kv_heads = n_kv_heads;
     a.max_pos = max_pos;
     return dispatch_decode<true>(a, n_heads, head_dim, workspace, (hipStream_t)stream);
+}
+
+int llm_attn_decode_rope_long(const uint16_t *qkv, uint16_t *kc, uint16_t *vc, uint16_t *out, int pos_host,
+                         const int32_t *pos_dev, const float *table, int n_heads, int n_kv_heads, int head_dim,
+                         int max_pos, void *workspace, llm_stream_t stream) {
+    LLM_REQUIRE(qkv && kc && vc && out && table && workspace, "llm_attn_decode_rope_long: null pointer");
+    LLM_REQUIRE(n_kv_heads > 0 && n_heads % n_kv_heads == 0, "llm_attn_decode_rope_long: heads %d/%d", n_heads, n_kv_heads);
+    LLM_REQUIRE(max_pos > 0 && max_pos % 64 == 0, "llm_attn_decode_rope_long: max_pos=%d must be a multiple of 64", max_pos);
+    LLM_REQUIRE(pos_dev || (pos_host >= 0 && pos_host < max_pos), "llm_attn_decode_rope_long: position %d of %d", pos_host,
+                max_pos);
+    LLM_REQUIRE(aligned16(qkv) && aligned16(kc) && aligned16(vc), "llm_attn_decode_rope_long: pointers must be 16-byte aligned");
+    AdArgs a = {};
+    a.q = (const half_t *)qkv;
+    a.kc = (half_t *)kc;
+    a.vc = (half_t *)vc;
+    a.out = (half_t *)out;
+    a.table = table;
+    a.pos_host = pos_host;
+    a.pos_dev = pos_dev;
+    a.n_kv_heads = n_kv_heads;
+    a.max_pos = max_pos;
+    return dispatch_decode_long<true>(a, n_heads, head_dim, workspace, (hipStream_t)stream);
 }
 
 } // extern "C"

@@ -210,8 +210,9 @@ def norm_lmhead_argmax(x, gain, w, eps=1e-5):
     return int(d_t.download()[0]), d_l.download()
 
 
-def attn_decode_rope(qkv, kc, vc, pos, n_heads, n_kv_heads, head_dim, theta=500000.0, repeats=1):
-    """Returns (out [Hq*hd], K cache, V cache) after rope + append + attention at position pos."""
+def attn_decode_rope(qkv, kc, vc, pos, n_heads, n_kv_heads, head_dim, theta=500000.0, repeats=1, long_form=False):
+    """Returns (out [Hq*hd], K cache, V cache) after rope + append + attention at position pos;
+    long_form selects the two-launch span/merge kernels."""
     qkv, kc, vc = _u16(qkv).reshape(-1), _u16(kc), _u16(vc)
     max_pos = kc.shape[1]
     d_q, d_k, d_v = DevBuf.from_host(qkv), DevBuf.from_host(kc), DevBuf.from_host(vc)
@@ -221,6 +222,7 @@ def attn_decode_rope(qkv, kc, vc, pos, n_heads, n_kv_heads, head_dim, theta=5000
     d_ws = DevBuf((wsb // 4,), np.uint32)
     d_ws.zero()
     for _ in range(repeats):
-        check(lib().llm_attn_decode_rope(d_q.ptr, d_k.ptr, d_v.ptr, d_o.ptr, pos, None, d_t.ptr, n_heads, n_kv_heads,
-                                         head_dim, max_pos, d_ws.ptr, None))
+        fn = lib().llm_attn_decode_rope_long if long_form else lib().llm_attn_decode_rope
+        check(fn(d_q.ptr, d_k.ptr, d_v.ptr, d_o.ptr, pos, None, d_t.ptr, n_heads, n_kv_heads,
+                 head_dim, max_pos, d_ws.ptr, None))
     return d_o.download(), d_k.download(), d_v.download()

@@ -50,9 +50,14 @@ struct Engine {
     int pos = 0;
     bool use_graph = true;
     bool sampling = false; // inference() samples like the reference instead of returning the argmax
-    llm_graph_t graph = nullptr;
+    // one captured decode step per attention form: [0] single launch (up to 512 cached positions),
+    // [1] span + merge launches (beyond)
+    llm_graph_t graph[2] = {nullptr, nullptr};
+    bool long_attn = false; // form used by the next decode step that is issued
     llm_event_t ev[4] = {nullptr, nullptr, nullptr, nullptr};
 };
+
+const int LONG_ATTN_FROM = 512; // cached positions from which the span + merge attention is faster
 
 Engine *eng(const CudaCache *c) {
     if (!c || !c->engine) llama3_fail("CudaCache was not created by init_cache");
@@ -133,8 +138,8 @@ void issue_pass(Engine *e, const Llama3 *m, int T, int pos0, bool dev_pos, bool 
                 llama3_check(llm_norm_linear(e->x, w.in_ln, c.rms_eps, w.wv, e->qkv + qd + kvd, kvd, d, s),
                              "llm_norm_linear(v)");
             }
-            llama3_check(llm_attn_decode_rope(e->qkv, kc, vc, e->attn, p0, pd, e->rope_table, Hq, Hkv, hd, c.max_pos,
-                                              e->ws_attn, s),
+            llama3_check((e->long_attn ? llm_attn_decode_rope_long : llm_attn_decode_rope)(
+                             e->qkv, kc, vc, e->attn, p0, pd, e->rope_table, Hq, Hkv, hd, c.max_pos, e->ws_attn, s),
                          "llm_attn_decode_rope");
             llama3_check(llm_linear(e->attn, qd, w.wo, e->x, d, e->x, d, 1, d, qd, s), "llm_linear(o)");
             llama3_check(llm_norm_linear_swiglu(e->x, w.post_ln, c.rms_eps, w.wg, w.wu, e->ffn, F, d, s),
@@ -180,9 +185,10 @@ void issue_pass(Engine *e, const Llama3 *m, int T, int pos0, bool dev_pos, bool 
 }
 
 void drop_graph(Engine *e) {
-    if (e->graph) {
-        llm_graph_destroy(e->graph);
-        e->graph = nullptr;
+    for (int f = 0; f < 2; ++f) {
+        if (!e->graph[f]) continue;
+        llm_graph_destroy(e->graph[f]);
+        e->graph[f] = nullptr;
     }
 }
 
@@ -218,6 +224,7 @@ int run_pass(Engine *e, const Llama3 *m, const int *tokens, int n) {
         }
         llama3_check(llm_memcpy_h2d(e->inject_dev, e->inject_host, sizeof(llm_half) * need, s), "H2D inject");
     }
+    e->long_attn = n == 1 && e->pos >= LONG_ATTN_FROM; // single rows go through the decode kernels
     issue_pass(e, m, n, e->pos, false, trace, inject);
     int32_t tok = -1;
     llama3_check(llm_memcpy_d2h(&tok, e->d_token, sizeof(int32_t), s), "D2H token");
@@ -233,15 +240,23 @@ int run_pass(Engine *e, const Llama3 *m, const int *tokens, int n) {
 }
 
 // One decode step from device state (d_tokens[*d_pos] in, next token out).
-void launch_decode_step(Engine *e, const Llama3 *m) {
+void capture_decode_graph(Engine *e, const Llama3 *m, int form) {
+    if (e->graph[form]) return;
+    e->long_attn = form == 1;
+    llama3_check(llm_graph_capture_begin(e->stream), "graph capture begin");
+    issue_pass(e, m, 1, 0, true, false);
+    llama3_check(llm_graph_capture_end(e->stream, &e->graph[form]), "graph capture end");
+}
+
+// pos: position of the token this step processes (known on the host although the kernels read it
+// from device memory), which selects the attention form
+void launch_decode_step(Engine *e, const Llama3 *m, int pos) {
+    const int form = pos >= LONG_ATTN_FROM ? 1 : 0;
     if (e->use_graph) {
-        if (!e->graph) {
-            llama3_check(llm_graph_capture_begin(e->stream), "graph capture begin");
-            issue_pass(e, m, 1, 0, true, false);
-            llama3_check(llm_graph_capture_end(e->stream, &e->graph), "graph capture end");
-        }
-        llama3_check(llm_graph_launch(e->graph, e->stream), "graph launch");
+        capture_decode_graph(e, m, form);
+        llama3_check(llm_graph_launch(e->graph[form], e->stream), "graph launch");
     } else {
+        e->long_attn = form == 1;
         issue_pass(e, m, 1, 0, true, false);
     }
 }
@@ -377,7 +392,7 @@ extern "C" int llama3_decode(Llama3 *m, CudaCache *C, int token) {
     llama3_check(llm_memcpy_h2d(e->d_tokens + e->pos, &t, sizeof(int32_t), s), "H2D token");
     llama3_check(llm_memcpy_h2d(e->d_pos, &p, sizeof(int32_t), s), "H2D position");
     llama3_check(llm_stream_sync(s), "stream sync");
-    launch_decode_step(e, m);
+    launch_decode_step(e, m, e->pos);
     int32_t tok = -1;
     llama3_check(llm_memcpy_d2h(&tok, e->d_token, sizeof(int32_t), s), "D2H token");
     llama3_check(llm_stream_sync(s), "stream sync");
@@ -399,13 +414,13 @@ extern "C" int llama3_generate(Llama3 *m, CudaCache *C, const int *prompt, int n
     int first = run_pass(e, m, prompt, n_prompt); // syncs
     llama3_check(llm_event_record(e->ev[1], s), "event record");
     // capture outside the timed decode region
-    if (e->use_graph && !e->graph && n_decode > 1) {
-        llama3_check(llm_graph_capture_begin(s), "graph capture begin");
-        issue_pass(e, m, 1, 0, true, false);
-        llama3_check(llm_graph_capture_end(s, &e->graph), "graph capture end");
+    if (e->use_graph && n_decode > 1) {
+        const int first_pos = start + n_prompt, last_pos = start + n_prompt + n_decode - 2;
+        if (first_pos < LONG_ATTN_FROM) capture_decode_graph(e, m, 0);
+        if (last_pos >= LONG_ATTN_FROM) capture_decode_graph(e, m, 1);
     }
     llama3_check(llm_event_record(e->ev[2], s), "event record");
-    for (int i = 1; i < n_decode; ++i) launch_decode_step(e, m);
+    for (int i = 1; i < n_decode; ++i) launch_decode_step(e, m, start + n_prompt + i - 1);
     llama3_check(llm_event_record(e->ev[3], s), "event record");
     llama3_check(llm_stream_sync(s), "stream sync");
     out_tokens[0] = first;

@@ -98,6 +98,42 @@ def test_reference_shaped_inference_call(gpu):
     model.close()
 
 
+def test_decode_across_the_long_context_attention_switch(gpu):
+    """Greedy decoding from position 500 to 560 changes attention kernels at 512 cached positions (one
+    launch before, span + merge launches after) and graphs with them: same ids with and without graphs,
+    same as stepping through the API, and the oracle agrees on hidden states on both sides."""
+    cfg = gpu.engine.config("tiny", max_pos=1024)
+    model = gpu.engine.Model.seeded(cfg, 21)
+    w = H.oracle_weights(model)
+    model.to_device()
+    prompt = gpu.engine.seeded_tokens(21, 500, cfg.vocab)
+    eng = gpu.engine.Engine(model, cfg, use_graph=True)
+    a, _ = eng.generate(prompt, 60)
+    eng.reset()
+    b, _ = eng.generate(prompt, 60)
+    eng.close()
+    eng2 = gpu.engine.Engine(model, cfg, use_graph=False)
+    c, _ = eng2.generate(prompt, 60)
+    assert list(a) == list(b) == list(c)
+    # step API with hidden states against the oracle, fed with the engine's own ids
+    o = orc.Model(H.cfg_dict(cfg), w, orc.ORC_REF16)
+    eng2.reset()
+    tok, _ = eng2.prefill(prompt)
+    tok_o, _, _ = o.forward(prompt)
+    assert tok == tok_o == a[0]
+    worst = 0.0
+    for i in range(1, 40):
+        t_g, h_g = eng2.decode(int(a[i - 1]), want_hidden=True)
+        t_o, h_o, lg_o = o.forward([int(a[i - 1])], want_hidden=True)
+        worst = max(worst, H.mixed_err(h_g, h_o), H.mixed_err(eng2.logits(), lg_o))
+        assert t_g == a[i]
+    say("long-context switch: worst err", worst)
+    assert worst <= H.TOL
+    o.close()
+    eng2.close()
+    model.close()
+
+
 def test_chunked_prompt_matches_single_pass(gpu):
     cfg, model, eng = _tiny_engine(gpu)
     prompt = gpu.engine.seeded_tokens(8, 50, cfg.vocab)

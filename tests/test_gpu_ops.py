@@ -409,3 +409,9 @@ def test_attn_decode_rope_fused(gpu, pos, max_pos, Hq, Hkv, hd):
     e = H.mixed_err(out, want)
     say("  err", e)
     assert e <= TOL
+    # the two-launch long-context form: same caches, same result to rounding, at every position
+    out_l, kc3, vc3 = gpu.ops.attn_decode_rope(qkv, kc, vc, pos, Hq, Hkv, hd, repeats=2, long_form=True)
+    assert np.array_equal(kc3, kc_ref) and np.array_equal(vc3, vc_ref)
+    e = H.mixed_err(out_l, want)
+    say("  long form err", e)
+    assert e <= TOL and H.mixed_err(out_l, out) <= TIGHT
