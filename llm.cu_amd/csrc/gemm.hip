@@ -318,21 +318,22 @@ template <int N> __device__ __forceinline__ void dma_wait_barrier() {
     asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(N) : "memory");
 }
 
-// (WGM*64) x (WGN*128) macro-tile, WGM*WGN wavefronts each owning 64 x 128 of it (NB = 2: 64 columns of
+// (WGM*FM*32) x (WGN*128) macro-tile, WGM*WGN wavefronts each owning (FM*32) x 128 of it (NB = 2: 64 columns of
 // gate and the same 64 of up), BK = 32, STAGES LDS buffers filled by direct global->LDS loads.
 // Split-K (ws != nullptr): workgroup (tile, z) covers k in [z*kper, (z+1)*kper) and stores its fp32
 // partial tile to ws[z][T][N]; splitk_reduce_kernel sums the slices in ascending z and finishes.
 // PREF: read the next tile's first fragments before the barrier (needs tiles kt and kt+1 landed at
 // barrier kt, so loads run STAGES-2 iterations ahead); otherwise loads run STAGES-1 ahead.
-template <int NB, int WGM, int WGN, int STAGES, bool PREF, int OCC>
+template <int NB, int WGM, int WGN, int STAGES, bool PREF, int OCC, int FM = 2>
 __global__ __launch_bounds__(WGM * WGN * 64, OCC) void gemm_dma_kernel(const half_t *__restrict__ x, int ldx,
                                                                const half_t *__restrict__ w, const half_t *__restrict__ w2,
                                                                const half_t *res, int ldr, half_t *out, int ldo, int T, int N, int K,
                                                                int tiles_m, int tiles_n, float *ws, int kper) {
     constexpr int NWAVES = WGM * WGN;
-    constexpr int BM = WGM * 64, BROWS = WGN * 128; // B rows in a stage (both matrices when NB = 2)
+    constexpr int WTM = FM * 32;                           // rows of a wave tile
+    constexpr int BM = WGM * WTM, BROWS = WGN * 128;       // B rows in a stage (both matrices when NB = 2)
     constexpr int BN = BROWS / NB;             // output columns per tile
-    constexpr int FM = 2, FN = 4 / NB;
+    constexpr int FN = 4 / NB;
     constexpr int STAGE_HALVES = (BM + BROWS) * DMA_BK;
     constexpr int LPT = (BM + BROWS) / 16 / NWAVES; // load instructions per wave per tile
     constexpr int AHEAD = PREF ? STAGES - 2 : STAGES - 1;
@@ -390,7 +391,7 @@ __global__ __launch_bounds__(WGM * WGN * 64, OCC) void gemm_dma_kernel(const hal
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks) {
         const int pc = (ks * 2 + lane / 32) ^ sw;
-        a_off[ks] = (wm * 64 + frow) * DMA_BK + pc * 8;
+        a_off[ks] = (wm * WTM + frow) * DMA_BK + pc * 8;
         b_off[ks] = BM * DMA_BK + ((NB == 1 ? wn * 128 : wn * 64) + frow) * DMA_BK + pc * 8;
     }
     half8_t af[2][FM], bf[2][4];
@@ -473,7 +474,7 @@ __global__ __launch_bounds__(WGM * WGN * 64, OCC) void gemm_dma_kernel(const hal
         float *wz = ws + (size_t)blockIdx.y * NB * T * N;
 #pragma unroll
         for (int i = 0; i < FM; ++i) {
-            const int m = m0 + wm * 64 + i * 32 + mrow;
+            const int m = m0 + wm * WTM + i * 32 + mrow;
 #pragma unroll
             for (int f = 0; f < 4; ++f)
 #pragma unroll
@@ -490,7 +491,7 @@ __global__ __launch_bounds__(WGM * WGN * 64, OCC) void gemm_dma_kernel(const hal
     }
 #pragma unroll
     for (int i = 0; i < FM; ++i) {
-        const int m = m0 + wm * 64 + i * 32 + mrow;
+        const int m = m0 + wm * WTM + i * 32 + mrow;
         const int mc = m < T ? m : T - 1;
 #pragma unroll
         for (int j = 0; j < FN; ++j) {
@@ -558,13 +559,13 @@ int gemm_init_workspace() {
     return LLM_OK;
 }
 
-template <int NB, int WGM, int WGN, int STAGES, bool PREF, int OCC>
+template <int NB, int WGM, int WGN, int STAGES, bool PREF, int OCC, int FM = 2>
 static int gemm_dma_launch(const half_t *x, int ldx, const half_t *w, const half_t *w2, const half_t *res, int ldr,
                            half_t *out, int ldo, int T, int N, int K, int splits, hipStream_t s) {
-    constexpr int BM = WGM * 64, BN = WGN * 128 / NB;
+    constexpr int BM = WGM * FM * 32, BN = WGN * 128 / NB;
     const int tiles_m = (T + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
     const size_t smem = sizeof(half_t) * (size_t)STAGES * (BM + WGN * 128) * DMA_BK;
-    auto kern = gemm_dma_kernel<NB, WGM, WGN, STAGES, PREF, OCC>;
+    auto kern = gemm_dma_kernel<NB, WGM, WGN, STAGES, PREF, OCC, FM>;
     static bool attr_set = false;
     if (!attr_set) {
         LLM_HIP_CHECK(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
@@ -648,7 +649,10 @@ int llm_linear(const uint16_t *x, int ldx, const uint16_t *w, const uint16_t *re
         return gemm_dma_launch<1, 4, 1, 3, false, 2>(xp, ldx, wp, nullptr, rp, ldr, op, ldo, T, N, K,
                                                      pick_splits(t4, T, N, K), s);
     }
-    return gemm_dma_launch<1, 4, 2, 4, true, 1>(xp, ldx, wp, nullptr, rp, ldr, op, ldo, T, N, K, 1, s);
+    // 256 x 256 tile as four waves of 128 x 128 (one per SIMD, accumulators in the second register
+    // file): a third fewer LDS reads per MFMA than eight waves of 64 x 128, which on this
+    // power-limited part is worth 3-12 % with real (non-constant) operands
+    return gemm_dma_launch<1, 2, 2, 4, true, 1, 4>(xp, ldx, wp, nullptr, rp, ldr, op, ldo, T, N, K, 1, s);
 }
 
 int llm_linear_swiglu(const uint16_t *x, int ldx, const uint16_t *wgate, const uint16_t *wup, uint16_t *out,
@@ -676,7 +680,7 @@ int llm_linear_swiglu(const uint16_t *x, int ldx, const uint16_t *wgate, const u
         return gemm_dma_launch<2, 2, 1, 4, false, 2>(xp, ldx, gp, up, nullptr, 0, op, ldo, T, N, K,
                                                      pick_splits(2 * (long)((N + 63) / 64), T, N, K, 2), s);
     if (T <= 1024) return gemm_dma_launch<2, 4, 1, 3, false, 2>(xp, ldx, gp, up, nullptr, 0, op, ldo, T, N, K, 1, s);
-    return gemm_dma_launch<2, 4, 2, 4, true, 1>(xp, ldx, gp, up, nullptr, 0, op, ldo, T, N, K, 1, s);
+    return gemm_dma_launch<2, 2, 2, 4, true, 1, 4>(xp, ldx, gp, up, nullptr, 0, op, ldo, T, N, K, 1, s);
 }
 
 int llm_norm_linear(const uint16_t *x, const uint16_t *gain, double eps, const uint16_t *w, uint16_t *out, int N, int K,
