@@ -141,6 +141,11 @@ ModelConfig llama3_config_tiny(void);
 CudaCache *init_cache_cfg(Llama3 *llama3_model, const ModelConfig *cfg);
 void free_cache(CudaCache *Cache);
 
+/* load_safetensor_weights() for every file followed by to_cuda(), streamed: headers first, then every
+ * tensor through two pinned 64 MiB buffers (read of one chunk overlaps the upload and BF16->FP16 of the
+ * previous), so host memory never holds the checkpoint.  Same device contents as the two-step path. */
+void load_safetensor_weights_streaming(Llama3 *llama3_model, const char *const *filenames, int n_files);
+
 /* KV-cached token loop.  prefill appends n tokens (any n >= 1) at the current
  * position and returns the greedy next token; decode appends one. */
 int llama3_prefill(Llama3 *m, CudaCache *c, const int *tokens, int n);

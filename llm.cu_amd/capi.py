@@ -132,6 +132,7 @@ HOST_ABI = {
     "_free_tensor": (None, [_TP]),
     "load_safetensor_weights": (None, [_LP, C.c_char_p]),
     "to_cuda": (None, [_LP]),
+    "load_safetensor_weights_streaming": (None, [_LP, C.POINTER(C.c_char_p), _i]),
     "init_cache": (_CP, [_LP]),
     "tokens_to_cuda": (C.POINTER(_i), [C.POINTER(_i), _i, _TP]),
     "inference": (_i, [_LP, _TP, C.POINTER(_i), C.POINTER(_i), _CP]),

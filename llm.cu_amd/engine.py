@@ -62,6 +62,16 @@ class Model:
             lib().load_safetensor_weights(m.handle, p.encode())
         return m
 
+    @classmethod
+    def from_files_streaming(cls, cfg, paths):
+        """Headers first, then every tensor through pinned staging buffers straight to the device."""
+        capi.require_gpu()
+        m = cls(cfg)
+        arr = (C.c_char_p * len(paths))(*[p.encode() for p in paths])
+        lib().load_safetensor_weights_streaming(m.handle, arr, len(paths))
+        m.on_device = True
+        return m
+
     def host_bf16(self):
         """dict of numpy views on the host bf16 payloads (valid until to_device)."""
         assert not self.on_device

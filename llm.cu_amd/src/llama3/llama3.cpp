@@ -152,14 +152,9 @@ void _m_component_tensor_operation(Llama3 *m, void (*f)(Tensor *)) {
     }
 }
 
-// to_cuda (src/llama3/llama3.cu:156-254): fp16 device storage for every
-// tensor, H2D of the bf16 payload, BF16->FP16 on the device, host payload
-// freed.  Differences in mechanism, not in result: one HBM slab instead of
-// four cudaMallocs per tensor (q/k/v and gate/up of a layer end up adjacent so
-// one projection launch covers them), one reusable bf16 staging buffer
-// instead of a malloc/free per tensor, and no device copies of
-// ndim/mem_len/shape (no kernel reads them).
-extern "C" void to_cuda(Llama3 *m) {
+// Lays every tensor out in one HBM slab (shapes must be known: mem_len set) and points d_fp16_tensor
+// into it.  Returns the element count of the largest tensor.
+size_t llama3_plan_slab(Llama3 *m) {
     std::vector<Tensor *> order; // slab order
     for (int i = 0; i < m->n_layers; ++i) {
         Llama3Layer *l = m->layers[i];
@@ -175,22 +170,38 @@ extern "C" void to_cuda(Llama3 *m) {
     size_t total = 0, largest = 0;
     std::vector<size_t> offs;
     for (Tensor *t : order) {
-        if (!t || !t->mem_len || !t->bf16_tensor)
+        if (!t || !t->mem_len || *t->mem_len <= 0)
             llama3_fail("to_cuda: a tensor was not loaded (missing from the checkpoint)");
         offs.push_back(total);
         size_t bytes = sizeof(llm_half) * (size_t)*t->mem_len;
         total += align_up(bytes, 256);
-        if (bytes > largest) largest = bytes;
+        if ((size_t)*t->mem_len > largest) largest = (size_t)*t->mem_len;
     }
-    void *slab = nullptr, *stage = nullptr;
+    void *slab = nullptr;
     llama3_check(llm_malloc(&slab, total), "llm_malloc(weight slab)");
-    llama3_check(llm_malloc(&stage, largest), "llm_malloc(bf16 staging)");
     {
         std::lock_guard<std::mutex> lk(g_mu);
         g_slabs.push_back({(char *)slab, total});
     }
     m->device_slab = slab;
     for (size_t i = 0; i < order.size(); ++i) order[i]->d_fp16_tensor = (llm_half *)((char *)slab + offs[i]);
+    return largest;
+}
+
+// to_cuda (src/llama3/llama3.cu:156-254): fp16 device storage for every
+// tensor, H2D of the bf16 payload, BF16->FP16 on the device, host payload
+// freed.  Differences in mechanism, not in result: one HBM slab instead of
+// four cudaMallocs per tensor (q/k/v and gate/up of a layer end up adjacent so
+// one projection launch covers them), one reusable bf16 staging buffer
+// instead of a malloc/free per tensor, and no device copies of
+// ndim/mem_len/shape (no kernel reads them).
+extern "C" void to_cuda(Llama3 *m) {
+    _m_component_tensor_operation(m, [](Tensor *t) {
+        if (!t || !t->bf16_tensor) llama3_fail("to_cuda: a tensor was not loaded (missing from the checkpoint)");
+    });
+    const size_t largest = llama3_plan_slab(m);
+    void *stage = nullptr;
+    llama3_check(llm_malloc(&stage, largest * sizeof(uint16_t)), "llm_malloc(bf16 staging)");
 
     // upload + convert in the reference's visitor order
     struct Ctx {

@@ -15,3 +15,7 @@ void _m_component_tensor_operation(Llama3 *llama3, void (*_func)(Tensor *));
 // True when p lies inside a weight slab owned by some Llama3 (such pointers
 // are released with the slab, not one by one).
 bool llama3_pointer_in_slab(const void *p);
+
+// One HBM slab for all tensors whose shapes are set; d_fp16_tensor of each points into it.  Returns the
+// element count of the largest tensor.
+size_t llama3_plan_slab(Llama3 *m);

@@ -52,17 +52,22 @@ int main(int argc, char **argv) {
     if (weights.empty()) {
         seeded_fill_model(model, &cfg, seed);
         printf("[CPU] Seeded synthetic weights (seed %llu)\n", (unsigned long long)seed);
+        to_cuda(model);
     } else {
+        // shards named on the command line (main.cu:73-76 loads four), streamed to the device
+        std::vector<std::string> names;
         size_t b = 0;
         while (b <= weights.size()) {
             size_t e = weights.find(',', b);
             if (e == std::string::npos) e = weights.size();
-            load_safetensor_weights(model, weights.substr(b, e - b).c_str());
+            names.push_back(weights.substr(b, e - b));
             b = e + 1;
         }
-        printf("[CPU] Loaded model to CPU\n");
+        std::vector<const char *> ptrs;
+        for (const std::string &n : names) ptrs.push_back(n.c_str());
+        load_safetensor_weights_streaming(model, ptrs.data(), (int)ptrs.size());
+        printf("[CPU] Read %d shard(s)\n", (int)ptrs.size());
     }
-    to_cuda(model);
     printf("[HIP] Loaded to the device, parameters converted to FP16\n");
     CudaCache *cache = init_cache_cfg(model, &cfg);
     llama3_set_use_graph(cache, graph);

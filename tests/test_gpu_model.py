@@ -134,6 +134,38 @@ def test_decode_across_the_long_context_attention_switch(gpu):
     model.close()
 
 
+def _all_device_tensors(model, cfg):
+    h = model.handle.contents
+    out = [model.device_fp16(h.embed_tokens), model.device_fp16(h.lm_head), model.device_fp16(h.norm)]
+    for l in range(cfg.n_layers):
+        L = h.layers[l].contents
+        for slot in ("input_layernorm", "mlp_down_proj", "mlp_gate_proj", "mlp_up_proj", "post_attention_layernorm",
+                     "self_attn_k_proj", "self_attn_o_proj", "self_attn_q_proj", "self_attn_v_proj"):
+            out.append(model.device_fp16(getattr(L, slot)))
+    return out
+
+
+@pytest.mark.parametrize("which", ["tiny", "8b-2-layers"])
+def test_streaming_load_equals_load_then_to_cuda(gpu, tmp_path, which):
+    """load_safetensor_weights_streaming() leaves the same fp16 bits on the device as the reference's
+    two steps; the 8B shapes make the embedding and LM head span 16 staging chunks each."""
+    import time
+    cfg = gpu.engine.config("tiny") if which == "tiny" else gpu.engine.config("8b", n_layers=2, max_pos=64)
+    path = str(tmp_path / "model.safetensors")
+    assert gpu.lib().seeded_write_safetensors(C.byref(cfg), 31, path.encode()) == 0
+    t0 = time.time()
+    a = gpu.engine.Model.from_files(cfg, [path]).to_device()
+    t1 = time.time()
+    b = gpu.engine.Model.from_files_streaming(cfg, [path])
+    t2 = time.time()
+    say("%s: %.1f MB file, load + to_cuda %.2f s, streaming %.2f s" % (which, os.path.getsize(path) / 1e6, t1 - t0, t2 - t1))
+    for x, y in zip(_all_device_tensors(a, cfg), _all_device_tensors(b, cfg)):
+        assert x.shape == y.shape and np.array_equal(x, y)
+    a.close()
+    b.close()
+    os.remove(path)
+
+
 def test_chunked_prompt_matches_single_pass(gpu):
     cfg, model, eng = _tiny_engine(gpu)
     prompt = gpu.engine.seeded_tokens(8, 50, cfg.vocab)

@@ -236,6 +236,18 @@ def test_missing_file_exits_1_with_the_reference_message():
     assert "An Error Occurred while opening /nonexistent/x.safetensors" in p.stdout
 
 
+def test_streaming_loader_reports_missing_files_and_missing_tensors(tmp_path):
+    code = ("import ctypes as C\nm = pkg.engine.Model(pkg.engine.config('tiny'))\n"
+            "arr = (C.c_char_p * 1)(%r.encode())\npkg.lib().load_safetensor_weights_streaming(m.handle, arr, 1)")
+    p = _child(code % "/nonexistent/x.safetensors")
+    assert p.returncode == 1 and "An Error Occurred while opening /nonexistent/x.safetensors" in p.stdout
+    # a checkpoint that lacks tensors of the model is refused before anything is allocated on a device
+    path = str(tmp_path / "partial.safetensors")
+    _write_safetensors(path, [("model.norm.weight", "BF16", (256,), np.zeros(256, np.uint16))])
+    p = _child(code % path)
+    assert p.returncode == 1 and "a tensor was not loaded" in p.stdout
+
+
 def test_unknown_tensor_name_exits_1(tmp_path):
     path = str(tmp_path / "bad.safetensors")
     _write_safetensors(path, [("model.layers.0.mystery.weight", "BF16", (4,), np.zeros(4, np.uint16))])
