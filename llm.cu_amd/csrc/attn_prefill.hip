@@ -83,7 +83,7 @@ __global__ __launch_bounds__(G *AP_QT * 64) void attn_prefill_kernel(const half_
     const int n_tiles = (pos0 + blk_last_q) / AP_BKEY + 1;
     const half_t *kbase = kc + (size_t)kvh * max_pos * HD;
     const half_t *vbase = vc + (size_t)kvh * HD * max_pos;
-    const float scale = 1.0f / sqrtf((float)HD);
+    const float c2 = 1.44269504088896341f / sqrtf((float)HD); // log2(e) / sqrt(hd)
     const int pm = (n & ~0xC) | ((n & 8) >> 1) | ((n & 4) << 1); // pi(n)
 
     half8_t rk[KL], rv[VL];
@@ -134,9 +134,11 @@ __global__ __launch_bounds__(G *AP_QT * 64) void attn_prefill_kernel(const half_
                 for (int s = 0; s < DS; ++s)
                     st[kh] = __builtin_amdgcn_mfma_f32_32x32x16_f16(load8(kr + 16 * s), qf[s], st[kh], 0, 0, 0);
             }
-            // scale, causal mask (only tiles that reach past the first row of this
-            // query tile need it), running max.  accumulator e of half kh is key
-            // key0 + 32*kh + 16*(e/8) + 8*hb + e%8.
+            // causal mask (only tiles that reach past the first row of this query tile need it) and
+            // running max on the raw scores.  accumulator e of half kh is key
+            // key0 + 32*kh + 16*(e/8) + 8*hb + e%8.  The softmax runs in base 2: with
+            // c = log2(e)/sqrt(hd), p = 2^(s*c - m) is one fma and one v_exp_f32 per score; a masked
+            // score (-FLT_MAX) gives 2^(-huge) = 0 without a select.
             float mx = -FLT_MAX;
             if (key0 + AP_BKEY - 1 > pos0 + q0) {
 #pragma unroll
@@ -144,8 +146,7 @@ __global__ __launch_bounds__(G *AP_QT * 64) void attn_prefill_kernel(const half_
 #pragma unroll
                     for (int e = 0; e < 16; ++e) {
                         const int key = key0 + 32 * kh + 16 * (e / 8) + 8 * hb + (e % 8);
-                        float sv = st[kh][e] * scale;
-                        sv = key <= qpos ? sv : -FLT_MAX;
+                        const float sv = key <= qpos ? st[kh][e] : -FLT_MAX;
                         st[kh][e] = sv;
                         mx = fmaxf(mx, sv);
                     }
@@ -153,32 +154,30 @@ __global__ __launch_bounds__(G *AP_QT * 64) void attn_prefill_kernel(const half_
 #pragma unroll
                 for (int kh = 0; kh < 2; ++kh)
 #pragma unroll
-                    for (int e = 0; e < 16; ++e) {
-                        const float sv = st[kh][e] * scale;
-                        st[kh][e] = sv;
-                        mx = fmaxf(mx, sv);
-                    }
+                    for (int e = 0; e < 16; ++e) mx = fmaxf(mx, st[kh][e]);
             }
             mx = fmaxf(mx, __shfl_xor(mx, 32));
-            const float m_new = fmaxf(m_run, mx);
-            const float alpha = __expf(m_run - m_new);
+            const float m_new = fmaxf(m_run, mx * c2);
+            const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
             float psum = 0.f;
 #pragma unroll
             for (int kh = 0; kh < 2; ++kh)
 #pragma unroll
                 for (int e = 0; e < 16; ++e) {
-                    const float sv = st[kh][e];
-                    const float p = sv == -FLT_MAX ? 0.f : __expf(sv - m_new);
+                    const float p = __builtin_amdgcn_exp2f(fmaf(st[kh][e], c2, -m_new));
                     st[kh][e] = p;
                     psum += p;
                 }
             psum += __shfl_xor(psum, 32);
             l_run = l_run * alpha + psum;
+            // the running max settles after the first tiles: skip the rescale of O^T when no lane needs it
+            if (__builtin_amdgcn_ballot_w64(m_new != m_run) != 0) {
+#pragma unroll
+                for (int t = 0; t < DT; ++t)
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) o[t][e] *= alpha;
+            }
             m_run = m_new;
-#pragma unroll
-            for (int t = 0; t < DT; ++t)
-#pragma unroll
-                for (int e = 0; e < 16; ++e) o[t][e] *= alpha;
 
             // O^T += V^T . P^T, four 16-key steps
 #pragma unroll
