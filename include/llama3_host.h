@@ -87,6 +87,20 @@ typedef struct {
     int index;
 } ProbIndex;
 
+/* src/tokenizer/tokenizer.cuh:14-32 */
+typedef struct TrieNode {
+    int _max_childs;
+    int child_len;
+    char *child_char;
+    struct TrieNode **child_node;
+    int token;
+} TrieNode;
+
+typedef struct {
+    TrieNode *root;
+    char **decode;
+} Llama3Tokenizer;
+
 /* ---- reference API ---------------------------------------------------- */
 Llama3 *init_llama3(int n_layers);
 void free_llama3(Llama3 *llama3);
@@ -110,7 +124,25 @@ int _compare_desc(const void *a, const void *b);
 int top_k_sampling(ProbIndex *prob_dist_array, int k);
 int top_p_sampling(ProbIndex *prob_dist_array, float p);
 
+/* Tokenizer, src/tokenizer/tokenizer.cuh:44-150: byte trie over the vocabulary, greedy longest match,
+ * decode table.  load_tokenizer() reads model_weights/modified_tokenizer.json as the reference does. */
+Llama3Tokenizer *load_tokenizer(void);
+int *tokenize(Llama3Tokenizer *tokenizer, char *input_str); /* [0] = count + 1, ids from [1], malloc'd */
+char *read_tokenizer_json(Llama3Tokenizer *tokenizer, const char *filename);
+long _get_file_size(const char *filename);
+TrieNode *init_trienode(void);
+void _build_trie(TrieNode *node, char *token_string, int token_int);
+int _find_child(TrieNode *node, char str, TrieNode **result);
+void _memexpand_child_nodes(TrieNode *node);
+void _build_decoder(char **decoder, char *token_string, int token_int);
+
 /* ---- extensions -------------------------------------------------------- */
+/* load_tokenizer() with the file and the decode-table size as arguments; release; the chat template
+ * of src/main.cu:26-59 around one user turn (malloc'd string). */
+Llama3Tokenizer *load_tokenizer_from(const char *filename, int decode_size);
+void free_tokenizer(Llama3Tokenizer *tokenizer, int decode_size);
+char *llama3_chat_prompt(const char *user_input);
+
 /* The reference fixes vocab 128256, temperature 0.7, top-k 50, top-p 0.9 at compile time
  * (inference.cu:24-29); init_cache_cfg() sets the vocabulary, this sets all four. */
 void llama3_sampler_config(int vocab, float temperature, int top_k, float top_p);

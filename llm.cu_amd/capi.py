@@ -156,6 +156,18 @@ HOST_ABI = {
     "seeded_fill_model": (None, [_LP, C.POINTER(ModelConfig), _u64]),
     "seeded_write_safetensors": (_i, [C.POINTER(ModelConfig), _u64, C.c_char_p]),
     "seeded_tensor_id": (_u64, [_i, _i]),
+    "load_tokenizer": (_vp, []),
+    "load_tokenizer_from": (_vp, [C.c_char_p, _i]),
+    "free_tokenizer": (None, [_vp, _i]),
+    "tokenize": (C.POINTER(_i), [_vp, C.c_char_p]),
+    "read_tokenizer_json": (_vp, [_vp, C.c_char_p]),
+    "_get_file_size": (C.c_long, [C.c_char_p]),
+    "init_trienode": (_vp, []),
+    "_build_trie": (None, [_vp, C.c_char_p, _i]),
+    "_find_child": (_i, [_vp, C.c_char, C.POINTER(_vp)]),
+    "_memexpand_child_nodes": (None, [_vp]),
+    "_build_decoder": (None, [_vp, C.c_char_p, _i]),
+    "llama3_chat_prompt": (_vp, [C.c_char_p]),
     "sample_next_token": (_i, [_vp, _vp]),
     "sample_next_token_reference": (_i, [_vp, _vp]),
     "temperature_softmax": (_vp, [_vp, _vp, C.c_float]),

@@ -4,6 +4,10 @@
 //
 //   llama3_main [--config tiny|8b] [--seed S] [--weights a.safetensors[,b,...]]
 //               [--prompt-len N] [--decode N] [--max-pos N] [--no-graph]
+//               [--tokenizer tokenizer.json --text "question" [--sample]]
+// With --tokenizer and --text the reference's chat turn runs instead (main.cu:98-130): chat template,
+// tokenize, inference() per token until a special id (>= 128000) or the context limit, decoded text
+// printed as it comes; --sample uses the reference's sampler instead of the argmax.
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -14,7 +18,8 @@
 #include "llmcu_hip.h"
 
 int main(int argc, char **argv) {
-    std::string config = "tiny", weights;
+    std::string config = "tiny", weights, tokenizer_path, text;
+    bool sample = false;
     uint64_t seed = 1234;
     int prompt_len = 16, decode = 32, max_pos = 0, graph = 1;
     for (int i = 1; i < argc; ++i) {
@@ -33,6 +38,9 @@ int main(int argc, char **argv) {
         else if (a == "--decode") decode = atoi(next());
         else if (a == "--max-pos") max_pos = atoi(next());
         else if (a == "--no-graph") graph = 0;
+        else if (a == "--tokenizer") tokenizer_path = next();
+        else if (a == "--text") text = next();
+        else if (a == "--sample") sample = true;
         else {
             printf("Error: unknown option %s\n", a.c_str());
             return 1;
@@ -71,6 +79,38 @@ int main(int argc, char **argv) {
     printf("[HIP] Loaded to the device, parameters converted to FP16\n");
     CudaCache *cache = init_cache_cfg(model, &cfg);
     llama3_set_use_graph(cache, graph);
+
+    if (!tokenizer_path.empty()) {
+        Llama3Tokenizer *tk = load_tokenizer_from(tokenizer_path.c_str(), cfg.vocab);
+        char *input = llama3_chat_prompt(text.c_str());
+        int *tokens = tokenize(tk, input);
+        const int limit = cfg.max_pos < 2048 ? cfg.max_pos : 2048;
+        llama3_set_sampling(cache, sample ? 1 : 0);
+        Tensor *X = (Tensor *)calloc(1, sizeof(Tensor));
+        int *d_tokens = tokens_to_cuda(tokens, cfg.d_model, X);
+        const int first_special = cfg.vocab > 128000 ? 128000 : cfg.vocab; // main.cu:113
+        int next_token = 0, produced = 0;
+        while (next_token < first_special && tokens[0] <= limit && produced < decode) {
+            next_token = inference(model, X, d_tokens, tokens, cache);
+            if (next_token < first_special && tk->decode[next_token]) {
+                printf("%s", tk->decode[next_token]);
+                fflush(stdout);
+            }
+            if (tokens[0] > 2048) break;
+            tokens[tokens[0]] = next_token;
+            tokens[0] = tokens[0] + 1;
+            ++produced;
+        }
+        printf("\n");
+        free(tokens);
+        free(input);
+        _free_tensor(X);
+        llm_free(d_tokens);
+        free_tokenizer(tk, cfg.vocab);
+        free_cache(cache);
+        free_llama3(model);
+        return 0;
+    }
 
     std::vector<int> prompt(prompt_len), out(decode);
     seeded_tokens(seed, prompt_len, cfg.vocab, prompt.data());

@@ -166,6 +166,35 @@ def test_streaming_load_equals_load_then_to_cuda(gpu, tmp_path, which):
     os.remove(path)
 
 
+def test_driver_chat_turn_with_tokenizer(gpu, tmp_path):
+    """llama3_main --tokenizer --text: the reference's chat turn (template, trie tokenizer, inference() per
+    token, decode table) end to end on the tiny model with a synthetic tokenizer.json; the ids it feeds are
+    checked by running the same prompt through the Python mirror."""
+    import subprocess
+    from tests.test_tokenizer import _write_tokenizer
+    from oracle import tokenizer_oracle as tok_orc
+    path = str(tmp_path / "tokenizer.json")
+    _write_tokenizer(path)
+    exe = os.path.join(os.path.dirname(gpu.capi.LIB_PATH), "llama3_main")
+    p = subprocess.run([exe, "--config", "tiny", "--max-pos", "256", "--tokenizer", path, "--text", "hi there",
+                        "--decode", "12", "--seed", "5"], capture_output=True, timeout=120)
+    assert p.returncode == 0, p.stdout + p.stderr
+    enc, dec = tok_orc.load_vocab(path)
+    prompt = (b"<|begin_of_text|><|start_header_id|>system<|end_header_id|>\n\nAs a helpful assistant, answer the user "
+              b"questions in detail and accurately\n<|eot_id|><|start_header_id|>user<|end_header_id|>\n\nhi there"
+              b"\n<|eot_id|><|start_header_id|>assistant<|end_header_id|>\n\n")
+    ids = tok_orc.tokenize(enc, prompt)
+    cfg = gpu.engine.config("tiny", max_pos=256)
+    model = gpu.engine.Model.seeded(cfg, 5).to_device()
+    eng = gpu.engine.Engine(model, cfg)
+    toks, _ = eng.generate(np.array(ids, np.int32), 12)
+    want = b"".join(dec.get(int(t), b"") for t in toks)
+    out = p.stdout.split(b"parameters converted to FP16\n", 1)[1]
+    assert out == want + b"\n", (out, want)
+    eng.close()
+    model.close()
+
+
 def test_chunked_prompt_matches_single_pass(gpu):
     cfg, model, eng = _tiny_engine(gpu)
     prompt = gpu.engine.seeded_tokens(8, 50, cfg.vocab)
