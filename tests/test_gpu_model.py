@@ -195,6 +195,38 @@ def test_driver_chat_turn_with_tokenizer(gpu, tmp_path):
     model.close()
 
 
+def test_sequence_limits(gpu):
+    """The cache can be filled to its last row (same ids as the oracle up to there); one row more, an id
+    outside the vocabulary or an empty call print the message and exit(1) as the reference's checks do."""
+    import subprocess
+    import sys
+    cfg = gpu.engine.config("tiny", max_pos=64)
+    model = gpu.engine.Model.seeded(cfg, 9)
+    w = H.oracle_weights(model)
+    model.to_device()
+    prompt = gpu.engine.seeded_tokens(9, 40, cfg.vocab)
+    eng = gpu.engine.Engine(model, cfg)
+    toks, _ = eng.generate(prompt, 25)      # rows 0..63 written: the cache is full
+    assert eng.pos == 64
+    o = orc.Model(H.cfg_dict(cfg), w, orc.ORC_REF16)
+    assert [int(t) for t in toks] == o.generate(prompt, 25)
+    o.close()
+    eng.close()
+    model.close()
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    head = ("import numpy as np, __graft_entry__ as g\npkg = g.load_package(); pkg.init(0)\n"
+            "cfg = pkg.engine.config('tiny', max_pos=64)\nm = pkg.engine.Model.seeded(cfg, 9).to_device()\n"
+            "e = pkg.engine.Engine(m, cfg)\np = pkg.engine.seeded_tokens(9, 40, cfg.vocab)\n")
+    for body, msg in (("e.generate(p, 25); e.decode(1)", "exceeds max_pos 64"),
+                      ("e.generate(p, 26)", "exceed max_pos 64"),
+                      ("e.prefill(np.arange(65, dtype=np.int32))", "exceeds max_pos 64"),
+                      ("e.prefill(np.array([5, 4096], np.int32))", "outside the vocabulary"),
+                      ("e.decode(-1)", "outside the vocabulary"),
+                      ("e.inference([])", "empty token list")):
+        r = subprocess.run([sys.executable, "-c", head + body], cwd=root, capture_output=True, text=True, timeout=120)
+        assert r.returncode == 1 and msg in r.stdout, (body, r.returncode, r.stdout[-300:], r.stderr[-300:])
+
+
 def test_chunked_prompt_matches_single_pass(gpu):
     cfg, model, eng = _tiny_engine(gpu)
     prompt = gpu.engine.seeded_tokens(8, 50, cfg.vocab)
