@@ -263,6 +263,46 @@ def test_llama3_8b_two_layers_parity(gpu):
     assert sum(a == b for a, b in zip(r["tokens_oracle"], r["tokens_gpu_forced"])) >= 7
 
 
+def test_llama3_8b_shapes_at_8k_context(gpu):
+    """8192-token prompt in one pass, then decode steps at positions 8192.. (the long-context attention
+    kernels, the large GEMM tiles and the KV cache at its real size), 8B layer shapes with 2 layers so that
+    the oracle's O(T^2) attention finishes in about a minute."""
+    cfg = gpu.engine.config("8b", n_layers=2, max_pos=8256)
+    model = gpu.engine.Model.seeded(cfg, 88)
+    w = H.oracle_weights(model)
+    model.to_device()
+    prompt = gpu.engine.seeded_tokens(88, 8192, cfg.vocab)
+    eng = gpu.engine.Engine(model, cfg, use_graph=False)
+    say("8K context: GPU prompt pass ...")
+    tok_g, hid_g = eng.prefill(prompt, want_hidden=True)
+    lg_g = eng.logits()
+    say("8K context: oracle prompt pass ...")
+    o = orc.Model(H.cfg_dict(cfg), w, orc.ORC_REF16)
+    tok_o, hid_o, lg_o = o.forward(prompt, want_hidden=True)
+    rows = np.r_[0:64, 4064:4128, 8128:8192]
+    e_h = [H.mixed_err(hid_g[l][rows], hid_o[l][rows]) for l in range(cfg.n_layers)]
+    e_all = H.mixed_err(hid_g, hid_o)
+    e_l = H.mixed_err(lg_g, lg_o)
+    say("8K context: hidden err", e_h, "all rows", e_all, "logits err", e_l, "tokens", tok_g, tok_o)
+    assert e_all <= H.TOL and e_l <= H.TOL
+    top = H.f16(lg_o)
+    assert tok_g == tok_o or float(top.max() - top[tok_g]) <= 2 * H.TOL * 8
+    # decode at ctx 8192.. on the oracle's ids
+    t = tok_o
+    for step in range(6):
+        t_g, h_g = eng.decode(int(t), want_hidden=True)
+        t_o, h_o, lg_o = o.forward([int(t)], want_hidden=True)
+        e = max(H.mixed_err(h_g, h_o), H.mixed_err(eng.logits(), lg_o))
+        top = H.f16(lg_o)
+        say("  step", step, "err", e, t_g, t_o)
+        assert e <= H.TOL
+        assert t_g == t_o or float(top.max() - top[t_g]) <= 2 * H.TOL * 8
+        t = t_o
+    o.close()
+    eng.close()
+    model.close()
+
+
 def _check_forced(r):
     tol = H.TOL
     assert r["convert_exact"]
