@@ -63,6 +63,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-steps", type=int, default=8)
     ap.add_argument("--no-graph", action="store_true")
+    ap.add_argument("--no-batch", action="store_true")
     a = ap.parse_args()
     if a.gpus != 1:
         sys.exit("bench.py: this build measures one MI355X; --gpus %d is not supported "
@@ -139,6 +140,31 @@ def main():
             % (1e3 / ms_l, 100 * prefill["decode_at_8k"]["hbm_frac"]))
     engine.close()
 
+    # ---- batched decode (beyond the reference, which serves one sequence): aggregate tokens/s --------
+    batched = None
+    if not a.no_batch:
+        batched = {}
+        bcfg = eng_mod.config("8b", max_pos=512)
+        for B in (4, 16):
+            engines = [eng_mod.Engine(model, bcfg, use_graph=False) for _ in range(B)]
+            cur = []
+            for b, e in enumerate(engines):
+                t, _ = e.prefill(eng_mod.seeded_tokens(a.seed + 10 + b, a.prompt, bcfg.vocab))
+                cur.append(t)
+            for _ in range(4):
+                cur = eng_mod.Engine.decode_batch(engines, cur)
+            pkg.capi.sync()
+            t0 = time.time()
+            n_steps = 32
+            for _ in range(n_steps):
+                cur = eng_mod.Engine.decode_batch(engines, cur)
+            pkg.capi.sync()
+            dt = time.time() - t0
+            batched[str(B)] = {"ms_per_step": 1e3 * dt / n_steps, "tok_per_s": B * n_steps / dt}
+            log("batched decode B=%d: %.2f ms per step, %.0f tok/s aggregate" % (B, 1e3 * dt / n_steps, B * n_steps / dt))
+            for e in engines:
+                e.close()
+
     # ---- CPU baseline: fp32 port of the reference forward pass on the host cores ---------------
     cpu = None
     if orc is not None:
@@ -172,7 +198,7 @@ def main():
                    "prompt_tokens": a.prompt, "decode_steps": K, "graph": not a.no_graph},
         "decode_hbm_frac": frac, "decode_bytes_per_token": decode_bytes(ctx_avg),
         "prompt_pass_ms": st.prefill_ms,
-        "roofline": roof, "cpu_baseline": cpu, "prefill_8k": prefill,
+        "roofline": roof, "cpu_baseline": cpu, "prefill_8k": prefill, "batched_decode": batched,
         "first_tokens": [int(t) for t in toks[:8]],
     }
     print(json.dumps(out), flush=True)

@@ -185,6 +185,13 @@ int llama3_decode(Llama3 *m, CudaCache *c, int token);
 void llama3_cache_reset(CudaCache *c);
 int llama3_cache_pos(const CudaCache *c);
 
+/* One decode step for `batch` (<= 16) independent sequences, each with its own cache (created with the
+ * same configuration, filled by llama3_prefill): tokens[b] is appended to sequence b, next_tokens[b]
+ * receives its greedy continuation.  Every weight matrix is streamed once per step for the whole batch.
+ * llama3_read_batch_logits copies the fp16 logits of sequence b of the last step (caches[0] of that step). */
+void llama3_decode_batch(Llama3 *m, CudaCache *const *caches, const int *tokens, int batch, int *next_tokens);
+void llama3_read_batch_logits(CudaCache *cache0, int b, llm_half *logits);
+
 typedef struct {
     double prefill_ms;     /* wall time of the prompt pass (HIP events) */
     double decode_ms;      /* wall time of all decode steps */

@@ -172,6 +172,14 @@ int llm_attn_decode_rope_long(const uint16_t *qkv_dev, uint16_t *k_cache_dev, ui
                          uint16_t *out_dev, int pos_host, const int32_t *pos_dev, const float *table_dev,
                          int n_heads, int n_kv_heads, int head_dim, int max_pos, void *workspace_dev,
                          llm_stream_t stream);
+/* The same step for `batch` (<= 16) independent sequences in one launch: row z of qkv_dev belongs to the
+ * sequence with caches k_caches[z], v_caches[z] (host arrays of device pointers) at position positions[z];
+ * workspace_dev holds batch * llm_attn_decode_workspace_bytes().  No counterpart in the reference (it
+ * serves one sequence). */
+int llm_attn_decode_rope_batch(const uint16_t *qkv_dev, int ldq, uint16_t *const *k_caches, uint16_t *const *v_caches,
+                               const int *positions, int batch, uint16_t *out_dev, int ldo, const float *table_dev,
+                               int n_heads, int n_kv_heads, int head_dim, int max_pos, void *workspace_dev,
+                               llm_stream_t stream);
 /* Same attention for T query rows at positions pos0..pos0+T-1 (prompt pass),
  * streaming softmax on MFMA tiles; never materialises [H,T,T].
  * q: [T, ldq] with head h at columns h*hd; out: [T, ldo].  Cache rows beyond

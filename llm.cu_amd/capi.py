@@ -116,6 +116,7 @@ HIP_ABI = {
     "llm_norm_linear": (_i, [_vp, _vp, C.c_double, _vp, _vp, _i, _i, _vp]),
     "llm_norm_linear_swiglu": (_i, [_vp, _vp, C.c_double, _vp, _vp, _vp, _i, _i, _vp]),
     "llm_attn_decode_rope": (_i, [_vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _vp, _vp]),
+    "llm_attn_decode_rope_batch": (_i, [_vp, _i, _vp, _vp, _vp, _i, _vp, _i, _vp, _i, _i, _i, _i, _vp, _vp]),
     "llm_attn_decode_rope_long": (_i, [_vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _vp, _vp]),
     "llm_norm_lmhead_argmax": (_i, [_vp, _vp, C.c_double, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp, _vp]),
     "llm_attn_decode_workspace_bytes": (_sz, [_i, _i]),
@@ -144,6 +145,8 @@ HOST_ABI = {
     "llama3_decode": (_i, [_LP, _CP, _i]),
     "llama3_cache_reset": (None, [_CP]),
     "llama3_cache_pos": (_i, [_CP]),
+    "llama3_decode_batch": (None, [_LP, C.POINTER(_CP), C.POINTER(_i), _i, C.POINTER(_i)]),
+    "llama3_read_batch_logits": (None, [_CP, _i, _vp]),
     "llama3_generate": (_i, [_LP, _CP, C.POINTER(_i), _i, _i, C.POINTER(_i), C.POINTER(GenStats)]),
     "llama3_set_hidden_trace": (None, [_CP, _vp]),
     "llama3_read_logits": (None, [_CP, _vp]),

@@ -368,8 +368,7 @@ __global__ __launch_bounds__(AD_THREADS) void attn_span_kernel(const AdArgs a) {
                                                          y == n_active - 1);
 }
 
-template <int HD, int G>
-__global__ __launch_bounds__(AD_MERGE_THREADS) void attn_merge_kernel(const AdArgs a) {
+template <int HD, int G> __device__ __forceinline__ void attn_merge_body(const AdArgs &a) {
     constexpr int PARTS = AD_MERGE_THREADS / HD;
     __shared__ float w[AD_MAX_SPLITS];
     __shared__ float red[2 * AD_MERGE_THREADS / 64];
@@ -429,6 +428,11 @@ __global__ __launch_bounds__(AD_MERGE_THREADS) void attn_merge_kernel(const AdAr
     }
 }
 
+template <int HD, int G>
+__global__ __launch_bounds__(AD_MERGE_THREADS) void attn_merge_kernel(const AdArgs a) {
+    attn_merge_body<HD, G>(a);
+}
+
 template <int HD, int G, bool FUSED>
 static int launch_decode_long(AdArgs a, void *ws, hipStream_t s) {
     const int Hq = a.n_kv_heads * G;
@@ -444,6 +448,97 @@ static int launch_decode_long(AdArgs a, void *ws, hipStream_t s) {
     LLM_LAUNCH_CHECK("attn_span_kernel");
     attn_merge_kernel<HD, G><<<dim3(Hq), dim3(AD_MERGE_THREADS), 0, s>>>(a);
     LLM_LAUNCH_CHECK("attn_merge_kernel");
+    return LLM_OK;
+}
+
+// ---------------------------------------------------------------------------
+// Batched decode: B independent sequences (each with its own KV cache and position) in one launch;
+// workgroup z serves sequence z with exactly the code of the single-sequence kernels.
+// ---------------------------------------------------------------------------
+#define AD_MAX_BATCH 16
+
+struct AdBatch {
+    const half_t *qkv; // [B][ldq] raw projection rows
+    int ldq;
+    half_t *out;       // [B][ldo]
+    int ldo;
+    half_t *kc[AD_MAX_BATCH], *vc[AD_MAX_BATCH];
+    int pos[AD_MAX_BATCH];
+    size_t ws_floats;  // workspace floats per sequence (long form)
+};
+
+__device__ __forceinline__ AdArgs ad_for_sequence(const AdArgs &common, const AdBatch &b, int z) {
+    AdArgs a = common;
+    a.q = b.qkv + (size_t)z * b.ldq;
+    a.out = b.out + (size_t)z * b.ldo;
+    a.kc = b.kc[z];
+    a.vc = b.vc[z];
+    a.pos_host = b.pos[z];
+    a.pos_dev = nullptr;
+    if (a.ws_acc) {
+        a.ws_acc += (size_t)z * b.ws_floats;
+        a.ws_ml += (size_t)z * b.ws_floats;
+    }
+    return a;
+}
+
+// every position below 512: the single-span form (dim-split workgroups, direct result)
+template <int HD, int G, int DSN>
+__global__ __launch_bounds__(AD_THREADS) void attn_decode_batch_kernel(const AdArgs common, const AdBatch b) {
+    __shared__ float sc[G * AD_LS];
+    __shared__ __attribute__((aligned(16))) half_t qs[G * HD];
+    __shared__ __attribute__((aligned(16))) half_t knew[HD];
+    __shared__ __attribute__((aligned(16))) half_t vnew[HD];
+    __shared__ float s_m[G], s_l[G];
+    __shared__ int s_last;
+    const AdArgs a = ad_for_sequence(common, b, blockIdx.z);
+    const int y = blockIdx.y;
+    attn_decode_body<HD, G, true, HD / DSN, AD_LS>(a, sc, qs, knew, vnew, s_m, s_l, &s_last, a.pos_host, 1, 0,
+                                                   y * (HD / DSN), y == 0);
+}
+
+template <int HD, int G>
+__global__ __launch_bounds__(AD_THREADS) void attn_span_batch_kernel(const AdArgs common, const AdBatch b) {
+    __shared__ float sc[G * AD_LONG_LS];
+    __shared__ __attribute__((aligned(16))) half_t qs[G * HD];
+    __shared__ __attribute__((aligned(16))) half_t knew[HD];
+    __shared__ __attribute__((aligned(16))) half_t vnew[HD];
+    __shared__ float s_m[G], s_l[G];
+    __shared__ int s_last;
+    const AdArgs a = ad_for_sequence(common, b, blockIdx.z);
+    const int n_active = a.pos_host / AD_LONG_LS + 1;
+    const int y = blockIdx.y;
+    if (y >= n_active) return;
+    attn_decode_body<HD, G, true, HD, AD_LONG_LS, true>(a, sc, qs, knew, vnew, s_m, s_l, &s_last, a.pos_host, n_active,
+                                                        y, 0, y == n_active - 1);
+}
+
+template <int HD, int G>
+__global__ __launch_bounds__(AD_MERGE_THREADS) void attn_merge_batch_kernel(const AdArgs common, const AdBatch b) {
+    attn_merge_body<HD, G>(ad_for_sequence(common, b, blockIdx.y));
+}
+
+template <int HD, int G>
+static int launch_decode_batch(AdArgs a, const AdBatch &b, int B, void *ws, hipStream_t s) {
+    constexpr int DSN = HD >= 128 ? 4 : 1;
+    const int Hq = a.n_kv_heads * G;
+    int max_pos_used = 0;
+    for (int z = 0; z < B; ++z) max_pos_used = b.pos[z] > max_pos_used ? b.pos[z] : max_pos_used;
+    if (max_pos_used < AD_LS) {
+        a.ws_acc = nullptr;
+        attn_decode_batch_kernel<HD, G, DSN><<<dim3(a.n_kv_heads, DSN, B), dim3(AD_THREADS), 0, s>>>(a, b);
+        LLM_LAUNCH_CHECK("attn_decode_batch_kernel");
+        return LLM_OK;
+    }
+    a.ws_acc = (float *)ws;
+    a.ws_ml = a.ws_acc + (size_t)Hq * AD_MAX_SPLITS * HD;
+    const int splits = (a.max_pos + AD_LONG_LS - 1) / AD_LONG_LS;
+    LLM_REQUIRE(splits <= AD_MAX_SPLITS, "llm_attn_decode_batch: max_pos=%d exceeds %d", a.max_pos, AD_MAX_SPLITS * AD_LONG_LS);
+    a.splits = splits;
+    attn_span_batch_kernel<HD, G><<<dim3(a.n_kv_heads, max_pos_used / AD_LONG_LS + 1, B), dim3(AD_THREADS), 0, s>>>(a, b);
+    LLM_LAUNCH_CHECK("attn_span_batch_kernel");
+    attn_merge_batch_kernel<HD, G><<<dim3(Hq, B), dim3(AD_MERGE_THREADS), 0, s>>>(a, b);
+    LLM_LAUNCH_CHECK("attn_merge_batch_kernel");
     return LLM_OK;
 }
 
@@ -536,6 +631,52 @@ int llm_attn_decode_rope_long(const uint16_t *qkv, uint16_t *kc, uint16_t *vc, u
     a.n_kv_heads = n_kv_heads;
     a.max_pos = max_pos;
     return dispatch_decode_long<true>(a, n_heads, head_dim, workspace, (hipStream_t)stream);
+}
+
+int llm_attn_decode_rope_batch(const uint16_t *qkv, int ldq, uint16_t *const *k_caches, uint16_t *const *v_caches,
+                               const int *positions, int batch, uint16_t *out, int ldo, const float *table,
+                               int n_heads, int n_kv_heads, int head_dim, int max_pos, void *workspace,
+                               llm_stream_t stream) {
+    LLM_REQUIRE(qkv && k_caches && v_caches && positions && out && table && workspace, "llm_attn_decode_rope_batch: null pointer");
+    LLM_REQUIRE(batch >= 1 && batch <= AD_MAX_BATCH, "llm_attn_decode_rope_batch: batch=%d (1..%d)", batch, AD_MAX_BATCH);
+    LLM_REQUIRE(n_kv_heads > 0 && n_heads % n_kv_heads == 0, "llm_attn_decode_rope_batch: heads %d/%d", n_heads, n_kv_heads);
+    LLM_REQUIRE(max_pos > 0 && max_pos % 64 == 0, "llm_attn_decode_rope_batch: max_pos=%d must be a multiple of 64", max_pos);
+    LLM_REQUIRE(ldq % 8 == 0 && ldq >= (n_heads + 2 * n_kv_heads) * head_dim && ldo >= n_heads * head_dim,
+                "llm_attn_decode_rope_batch: ldq=%d ldo=%d", ldq, ldo);
+    LLM_REQUIRE(aligned16(qkv), "llm_attn_decode_rope_batch: qkv must be 16-byte aligned");
+    AdBatch b = {};
+    b.qkv = (const half_t *)qkv;
+    b.ldq = ldq;
+    b.out = (half_t *)out;
+    b.ldo = ldo;
+    b.ws_floats = llm_attn_decode_workspace_bytes(n_heads, head_dim) / sizeof(float);
+    for (int z = 0; z < batch; ++z) {
+        LLM_REQUIRE(k_caches[z] && v_caches[z] && aligned16(k_caches[z]) && aligned16(v_caches[z]),
+                    "llm_attn_decode_rope_batch: cache %d", z);
+        LLM_REQUIRE(positions[z] >= 0 && positions[z] < max_pos, "llm_attn_decode_rope_batch: position %d of %d",
+                    positions[z], max_pos);
+        b.kc[z] = (half_t *)k_caches[z];
+        b.vc[z] = (half_t *)v_caches[z];
+        b.pos[z] = positions[z];
+    }
+    AdArgs a = {};
+    a.table = table;
+    a.n_kv_heads = n_kv_heads;
+    a.max_pos = max_pos;
+    const int G = n_heads / n_kv_heads;
+    hipStream_t s = (hipStream_t)stream;
+#define AD_CASE(HD_, G_) \
+    if (head_dim == HD_ && G == G_) return launch_decode_batch<HD_, G_>(a, b, batch, workspace, s);
+    AD_CASE(128, 4)
+    AD_CASE(128, 8)
+    AD_CASE(128, 1)
+    AD_CASE(64, 4)
+    AD_CASE(64, 1)
+    AD_CASE(32, 4)
+    AD_CASE(32, 1)
+#undef AD_CASE
+    llm_set_error("llm_attn_decode_rope_batch: head_dim=%d with group size %d is not built", head_dim, G);
+    return LLM_ERR_INVALID;
 }
 
 } // extern "C"

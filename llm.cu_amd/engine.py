@@ -165,6 +165,21 @@ class Engine:
         arr[1:n + 1] = tokens
         return lib().inference(self.model.handle, None, None, arr.ctypes.data_as(C.POINTER(C.c_int)), self.cache)
 
+    @staticmethod
+    def decode_batch(engines, tokens):
+        """One step for several sequences (one Engine each, same model and configuration); returns the greedy ids."""
+        B = len(engines)
+        caches = (capi.HOST_ABI["init_cache"][0] * B)(*[e.cache for e in engines])
+        tok = (C.c_int * B)(*[int(t) for t in tokens])
+        out = (C.c_int * B)()
+        lib().llama3_decode_batch(engines[0].model.handle, caches, tok, B, out)
+        return [int(x) for x in out]
+
+    def batch_logits(self, b):
+        out = np.empty(self.cfg.vocab, np.uint16)
+        lib().llama3_read_batch_logits(self.cache, b, out.ctypes.data)
+        return out
+
     def set_sampling(self, on):
         """inference() returns the reference's temperature/top-k/top-p sample (True) or the argmax (False)."""
         lib().llama3_set_sampling(self.cache, 1 if on else 0)

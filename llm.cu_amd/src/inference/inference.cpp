@@ -54,6 +54,11 @@ struct Engine {
     // [1] span + merge launches (beyond)
     llm_graph_t graph[2] = {nullptr, nullptr};
     bool long_attn = false; // form used by the next decode step that is issued
+    // scratch of llama3_decode_batch (allocated by the first call on this cache as sequence 0)
+    int batch_cap = 0;
+    llm_half *b_logits = nullptr; // [batch][vocab]
+    int32_t *b_ids = nullptr;     // [batch] input ids, then the argmax results
+    void *b_ws_attn = nullptr;
     llm_event_t ev[4] = {nullptr, nullptr, nullptr, nullptr};
 };
 
@@ -340,7 +345,8 @@ extern "C" void free_cache(CudaCache *C) {
         llm_stream_sync(e->stream);
         drop_graph(e);
         void *bufs[] = {e->x, e->xn, e->qkv, e->attn, e->ffn, e->logits, e->kc, e->vc, e->rope_table,
-                        e->d_tokens, e->d_pos, e->d_token, e->ws_attn, e->ws_lm, e->trace_dev, e->inject_dev};
+                        e->d_tokens, e->d_pos, e->d_token, e->ws_attn, e->ws_lm, e->trace_dev, e->inject_dev,
+                        e->b_logits, e->b_ids, e->b_ws_attn};
         for (void *b : bufs) llm_free(b);
         for (auto ev : e->ev) llm_event_destroy(ev);
         llm_stream_destroy(e->stream);
@@ -443,6 +449,98 @@ extern "C" int llama3_generate(Llama3 *m, CudaCache *C, const int *prompt, int n
         stats->n_decode_steps = n_decode - 1;
     }
     return 0;
+}
+
+// ---------------------------------------------------------------------------
+// One decode step for `batch` independent sequences (no counterpart in the reference, which serves one):
+// the activations of all sequences form a [batch, d] matrix, so every weight matrix is streamed once per
+// step for all of them (the 2..16-row MFMA kernel that reads weights once), while each sequence keeps its
+// own KV cache and position.  caches[0] lends its activation buffers.  Per-row arithmetic is that of a
+// one-token prompt pass (separate RMSNorm, same rounding points as the single-sequence step).
+// ---------------------------------------------------------------------------
+extern "C" void llama3_decode_batch(Llama3 *m, CudaCache *const *caches, const int *tokens, int batch, int *next_tokens) {
+    if (batch < 1 || batch > 16) llama3_fail("llama3_decode_batch: batch %d (1..16)", batch);
+    Engine *e0 = eng(caches[0]);
+    const ModelConfig &c = e0->cfg;
+    const int d = c.d_model, hd = c.head_dim, Hq = c.n_heads, Hkv = c.n_kv_heads, F = c.ffn_dim;
+    const int qd = Hq * hd, kvd = Hkv * hd, QKV = e0->qkv_dim;
+    llm_stream_t s = e0->stream;
+    Engine *es[16];
+    int pos[16];
+    for (int b = 0; b < batch; ++b) {
+        es[b] = eng(caches[b]);
+        for (int a = 0; a < b; ++a)
+            if (es[a] == es[b]) llama3_fail("llama3_decode_batch: sequence %d and %d share a cache", a, b);
+        const ModelConfig &cb = es[b]->cfg;
+        if (cb.max_pos != c.max_pos || cb.d_model != d || cb.n_layers != c.n_layers || cb.vocab != c.vocab)
+            llama3_fail("llama3_decode_batch: cache %d has a different configuration", b);
+        if (es[b]->pos + 1 > c.max_pos) llama3_fail("sequence of %d tokens exceeds max_pos %d", es[b]->pos + 1, c.max_pos);
+        if (tokens[b] < 0 || tokens[b] >= c.vocab) llama3_fail("token id %d outside the vocabulary", tokens[b]);
+        pos[b] = es[b]->pos;
+        if (b > 0) llama3_check(llm_stream_sync(es[b]->stream), "stream sync"); // its prompt pass has finished
+    }
+    if (c.max_pos < batch) llama3_fail("llama3_decode_batch: max_pos %d below the batch size", c.max_pos);
+    if (e0->batch_cap < batch) {
+        if (e0->b_logits) llm_free(e0->b_logits);
+        if (e0->b_ids) llm_free(e0->b_ids);
+        if (e0->b_ws_attn) llm_free(e0->b_ws_attn);
+        e0->b_logits = dmalloc<llm_half>((size_t)16 * c.vocab, "llm_malloc(batch logits)");
+        e0->b_ids = dmalloc<int32_t>(16, "llm_malloc(batch ids)");
+        const size_t wsb = llm_attn_decode_workspace_bytes(Hq, hd);
+        e0->b_ws_attn = dmalloc<char>(wsb * 16, "llm_malloc(batch attention workspace)");
+        llama3_check(llm_fill_zero(e0->b_ws_attn, wsb * 16, s), "zero workspace");
+        e0->batch_cap = 16;
+    }
+    llama3_check(llm_memcpy_h2d(e0->b_ids, tokens, sizeof(int32_t) * (size_t)batch, s), "H2D ids");
+    llama3_check(llm_embed_gather(m->embed_tokens->d_fp16_tensor, e0->b_ids, nullptr, e0->x, batch, d, c.vocab, s),
+                 "llm_embed_gather");
+    for (int l = 0; l < c.n_layers; ++l) {
+        const LayerW w = layer_w(m, l);
+        uint16_t *kcs[16], *vcs[16];
+        for (int b = 0; b < batch; ++b) {
+            kcs[b] = es[b]->kc + (size_t)l * es[b]->kv_layer_elems;
+            vcs[b] = es[b]->vc + (size_t)l * es[b]->kv_layer_elems;
+        }
+        llama3_check(llm_rmsnorm(e0->x, w.in_ln, e0->xn, batch, d, c.rms_eps, s), "llm_rmsnorm");
+        if (w.wk == w.wq + (size_t)qd * d && w.wv == w.wk + (size_t)kvd * d) {
+            llama3_check(llm_linear(e0->xn, d, w.wq, nullptr, 0, e0->qkv, QKV, batch, QKV, d, s), "llm_linear(qkv)");
+        } else {
+            llama3_check(llm_linear(e0->xn, d, w.wq, nullptr, 0, e0->qkv, QKV, batch, qd, d, s), "llm_linear(q)");
+            llama3_check(llm_linear(e0->xn, d, w.wk, nullptr, 0, e0->qkv + qd, QKV, batch, kvd, d, s), "llm_linear(k)");
+            llama3_check(llm_linear(e0->xn, d, w.wv, nullptr, 0, e0->qkv + qd + kvd, QKV, batch, kvd, d, s), "llm_linear(v)");
+        }
+        llama3_check(llm_attn_decode_rope_batch(e0->qkv, QKV, kcs, vcs, pos, batch, e0->attn, qd, e0->rope_table, Hq, Hkv,
+                                                hd, c.max_pos, e0->b_ws_attn, s),
+                     "llm_attn_decode_rope_batch");
+        llama3_check(llm_linear(e0->attn, qd, w.wo, e0->x, d, e0->x, d, batch, d, qd, s), "llm_linear(o)");
+        llama3_check(llm_rmsnorm(e0->x, w.post_ln, e0->xn, batch, d, c.rms_eps, s), "llm_rmsnorm");
+        llama3_check(llm_linear_swiglu(e0->xn, d, w.wg, w.wu, e0->ffn, F, batch, F, d, s), "llm_linear_swiglu");
+        llama3_check(llm_linear(e0->ffn, F, w.wd, e0->x, d, e0->x, d, batch, d, F, s), "llm_linear(down)");
+    }
+    llama3_check(llm_rmsnorm(e0->x, m->norm->d_fp16_tensor, e0->xn, batch, d, c.rms_eps, s), "llm_rmsnorm");
+    llama3_check(llm_linear(e0->xn, d, m->lm_head->d_fp16_tensor, nullptr, 0, e0->b_logits, c.vocab, batch, c.vocab, d, s),
+                 "llm_linear(lm_head)");
+    for (int b = 0; b < batch; ++b)
+        llama3_check(llm_argmax_f16(e0->b_logits + (size_t)b * c.vocab, c.vocab, e0->b_ids + b, e0->ws_lm, s),
+                     "llm_argmax_f16");
+    int32_t out[16];
+    llama3_check(llm_memcpy_d2h(out, e0->b_ids, sizeof(int32_t) * (size_t)batch, s), "D2H tokens");
+    llama3_check(llm_stream_sync(s), "stream sync");
+    for (int b = 0; b < batch; ++b) {
+        next_tokens[b] = (int)out[b];
+        es[b]->tokens.push_back(tokens[b]);
+        es[b]->pos += 1;
+    }
+}
+
+// fp16 logits of sequence b after the last llama3_decode_batch() in which caches[0] was this cache
+extern "C" void llama3_read_batch_logits(CudaCache *C0, int b, llm_half *logits) {
+    Engine *e = eng(C0);
+    if (!e->b_logits || b < 0 || b >= e->batch_cap) llama3_fail("llama3_read_batch_logits: no batch step has run");
+    llama3_check(llm_memcpy_d2h(logits, e->b_logits + (size_t)b * e->cfg.vocab, sizeof(llm_half) * (size_t)e->cfg.vocab,
+                                e->stream),
+                 "D2H logits");
+    llama3_check(llm_stream_sync(e->stream), "stream sync");
 }
 
 extern "C" void llama3_set_hidden_trace(CudaCache *C, llm_half *hidden) { eng(C)->trace_host = hidden; }

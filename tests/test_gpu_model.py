@@ -195,6 +195,50 @@ def test_driver_chat_turn_with_tokenizer(gpu, tmp_path):
     model.close()
 
 
+@pytest.mark.parametrize("lens", [[5], [7, 40, 3, 21], [500, 20, 515, 9, 64, 130, 2, 33, 77, 5, 6, 90, 100, 250, 11, 12]])
+def test_batched_decode_matches_independent_sequences(gpu, lens):
+    """llama3_decode_batch: sequences of different lengths (one crossing 512 cached positions, which switches
+    the whole launch to the span + merge attention) advance together; each must follow its own oracle."""
+    cfg = gpu.engine.config("tiny", max_pos=1024)
+    model = gpu.engine.Model.seeded(cfg, 17)
+    w = H.oracle_weights(model)
+    model.to_device()
+    B = len(lens)
+    engines = [gpu.engine.Engine(model, cfg, use_graph=False) for _ in range(B)]
+    oracles = [orc.Model(H.cfg_dict(cfg), w, orc.ORC_REF16) for _ in range(B)]
+    cur = []
+    for b, n in enumerate(lens):
+        prompt = gpu.engine.seeded_tokens(100 + b, n, cfg.vocab)
+        t_g, _ = engines[b].prefill(prompt)
+        t_o, _, _ = oracles[b].forward(prompt)
+        assert t_g == t_o
+        cur.append(t_o)
+    worst = 0.0
+    for step in range(14):
+        nxt = gpu.engine.Engine.decode_batch(engines, cur)
+        new = []
+        for b in range(B):
+            t_o, _, lg_o = oracles[b].forward([cur[b]])
+            e = H.mixed_err(engines[0].batch_logits(b), lg_o)
+            worst = max(worst, e)
+            top = H.f16(lg_o)
+            assert nxt[b] == t_o or float(top.max() - top[nxt[b]]) <= 2 * H.TOL * 8, (step, b, nxt[b], t_o)
+            new.append(t_o)
+        cur = new
+        assert [e.pos for e in engines] == [n + step + 1 for n in lens]
+    say("batched decode", B, "worst logits err", worst)
+    assert worst <= H.TOL
+    # a sequence can go on alone afterwards: the single-sequence step sees the rows the batch appended
+    t_g, _ = engines[-1].decode(cur[-1])
+    t_o, _, _ = oracles[-1].forward([cur[-1]])
+    assert t_g == t_o
+    for e in engines:
+        e.close()
+    for o in oracles:
+        o.close()
+    model.close()
+
+
 def test_sequence_limits(gpu):
     """The cache can be filled to its last row (same ids as the oracle up to there); one row more, an id
     outside the vocabulary or an empty call print the message and exit(1) as the reference's checks do."""
