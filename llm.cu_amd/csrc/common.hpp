@@ -98,6 +98,11 @@ __device__ __forceinline__ float dot8(half8_t a, half8_t b, float acc) {
 }
 
 __device__ __forceinline__ half8_t load8(const half_t *p) { return *reinterpret_cast<const half8_t *>(p); }
+// streamed once: do not keep the line in the caches
+__device__ __forceinline__ half8_t load8_nt(const half_t *p) {
+    uint4_t v = __builtin_nontemporal_load(reinterpret_cast<const uint4_t *>(p));
+    return __builtin_bit_cast(half8_t, v);
+}
 __device__ __forceinline__ void store8(half_t *p, half8_t v) { *reinterpret_cast<half8_t *>(p) = v; }
 
 // fp16 result with an optional residual: the reference stores the projection

@@ -48,26 +48,39 @@ __global__ __launch_bounds__(SK_WAVES * 64) void skinny_kernel(const half_t *__r
     const half_t *wp = w + (size_t)nrow * K + kbeg + 8 * g;
     const half_t *wp2 = SWIGLU ? w2 + (size_t)nrow * K + kbeg + 8 * g : nullptr;
     float4_t acc = {0.f, 0.f, 0.f, 0.f}, acc2 = {0.f, 0.f, 0.f, 0.f};
+    // Weights are read once (non-temporal), U k-steps per round; the loads of round i+1 are issued
+    // before the MFMAs of round i (two register sets), so a wave always has a round in flight.
     constexpr int U = 4;
-    int k = 0;
-    for (; k + 32 * U <= kslice; k += 32 * U) {
-        half8_t a[U], b[U], b2[U];
+    half8_t a[2][U], b[2][U], b2[2][U];
+    const int rounds = kslice / (32 * U);
+    auto fetch = [&](int set, int k) {
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            b[u] = load8(wp + k + 32 * u);
-            if (SWIGLU) b2[u] = load8(wp2 + k + 32 * u);
-            a[u] = load8(xp + k + 32 * u);
+            b[set][u] = load8_nt(wp + k + 32 * u);
+            if (SWIGLU) b2[set][u] = load8_nt(wp2 + k + 32 * u);
+            a[set][u] = load8(xp + k + 32 * u);
         }
+    };
+    auto mma = [&](int set) {
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[u], b[u], acc, 0, 0, 0);
-            if (SWIGLU) acc2 = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[u], b2[u], acc2, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[set][u], b[set][u], acc, 0, 0, 0);
+            if (SWIGLU) acc2 = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[set][u], b2[set][u], acc2, 0, 0, 0);
         }
+    };
+    if (rounds > 0) fetch(0, 0);
+    int rd = 0;
+    for (; rd + 2 <= rounds; rd += 2) { // unrolled by two so that the register-set index is a constant
+        fetch(1, (rd + 1) * 32 * U);
+        mma(0);
+        if (rd + 2 < rounds) fetch(0, (rd + 2) * 32 * U);
+        mma(1);
     }
-    for (; k < kslice; k += 32) {
-        half8_t a = load8(xp + k), b = load8(wp + k);
-        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, acc, 0, 0, 0);
-        if (SWIGLU) acc2 = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, load8(wp2 + k), acc2, 0, 0, 0);
+    if (rd < rounds) mma(0);
+    for (int k = rounds * 32 * U; k < kslice; k += 32) {
+        half8_t av = load8(xp + k), bv = load8(wp + k);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, bv, acc, 0, 0, 0);
+        if (SWIGLU) acc2 = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, load8(wp2 + k), acc2, 0, 0, 0);
     }
 #pragma unroll
     for (int i = 0; i < 4; ++i) {

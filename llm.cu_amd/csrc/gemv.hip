@@ -36,11 +36,6 @@ struct GemvArgs {
     int N, K, rpw;
 };
 
-__device__ __forceinline__ half8_t load8_nt(const half_t *p) {
-    uint4_t v = __builtin_nontemporal_load(reinterpret_cast<const uint4_t *>(p));
-    return __builtin_bit_cast(half8_t, v);
-}
-
 __device__ __forceinline__ float silu_f(float g) { return g / (1.0f + expf(-g)); }
 
 // Candidates are packed (order key + 1) << 32 | ~index so that an unsigned max
