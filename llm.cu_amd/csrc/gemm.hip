@@ -14,6 +14,7 @@
 //   32x32x16: A lane l -> row l%32, k = 8*(l/32)..+7;  B lane l -> col l%32, same k;
 //             D lane l -> col l%32, rows 8*(i/4) + 4*(l/32) + i%4, i<16.
 #include <cmath>
+#include <type_traits>
 
 #include "common.hpp"
 
@@ -23,6 +24,10 @@ int gemv_swiglu_launch(const half_t *x, const half_t *gain, double eps, const ha
                        half_t *out, int N, int K, hipStream_t s);
 
 __device__ __forceinline__ float silu_g(float g) { return g / (1.0f + expf(-g)); }
+
+// address-space casts for __builtin_amdgcn_global_load_lds (global memory straight into LDS)
+#define DMA_GP(p) ((const __attribute__((address_space(1))) void *)(p))
+#define DMA_LP(p) ((__attribute__((address_space(3))) void *)(p))
 
 // ---------------------------------------------------------------------------
 // skinny
@@ -108,6 +113,156 @@ __global__ __launch_bounds__(SK_WAVES * 64) void skinny_kernel(const half_t *__r
             }
         }
     }
+}
+
+// ---------------------------------------------------------------------------
+// skinny, weights through LDS
+// ---------------------------------------------------------------------------
+// The kernel above reads, per load instruction, 64 bytes from each of 16 weight rows.  Here every wave
+// instruction moves 512 contiguous bytes of two rows straight into the wave's own LDS tile
+// (global_load_lds), i.e. the DRAM pattern of the GEMV, and the MFMA fragments are read back from LDS.
+// Same work split: workgroup = 16 output columns, WAVES wavefronts each own a k-slice and process it in
+// chunks of 256; two chunks per wave are in LDS, one being consumed while the next lands (no workgroup
+// barrier: the tiles are private to the wave).  Lane l of an instruction fetches 16-byte chunk
+// (l%32) ^ (row&15) of its row so that the 16 rows a fragment read touches per cycle sit in 16
+// different bank groups.
+#define SKD_CHUNK 256
+
+template <bool SWIGLU, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void skinny_dma_kernel(const half_t *__restrict__ x, int ldx,
+                                                                const half_t *__restrict__ w,
+                                                                const half_t *__restrict__ w2, const half_t *res,
+                                                                int ldr, half_t *out, int ldo, int T, int N, int K) {
+    constexpr int NW = SWIGLU ? 2 : 1;
+    constexpr int TILE = 16 * SKD_CHUNK;              // halves per weight tile (8 KB)
+    constexpr int VM_PER_CHUNK = 8 * NW + 8;          // load instructions a chunk issues (weights + x)
+    extern __shared__ __attribute__((aligned(16))) half_t sk_lds[]; // [WAVES][2 stages][NW][TILE]
+    __shared__ float red[NW][WAVES][64][4];
+    const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
+    const int r = lane % 16, g = lane / 16;
+    const int mrow = r < T ? r : T - 1;
+    const int kslice = K / WAVES; // multiple of SKD_CHUNK
+    const int kbeg = wave * kslice;
+    const int nchunks = kslice / SKD_CHUNK;
+    half_t *mine = sk_lds + (size_t)wave * 2 * NW * TILE;
+    // The workgroup walks over column tiles blockIdx.x, blockIdx.x + gridDim.x, ...; its waves see one
+    // flat sequence of (tile, chunk) items, so the first chunk of the next tile is already on its way
+    // while the last chunk of the current one is consumed and reduced.
+    const int n_tiles = (N + 15) / 16;
+    const int my_tiles = ((int)blockIdx.x < n_tiles) ? (n_tiles - 1 - (int)blockIdx.x) / (int)gridDim.x + 1 : 0;
+    const int n_items = my_tiles * nchunks;
+
+    const int lrow = lane / 32, lpos = lane % 32;
+    const half_t *xp = x + (size_t)mrow * ldx + kbeg + 8 * g;
+    half8_t a[2][8];
+    auto issue = [&](int item) {
+        const int tile = blockIdx.x + (item / nchunks) * gridDim.x, chunk = item % nchunks;
+        half_t *st = mine + (size_t)(item & 1) * NW * TILE;
+        const int k0 = kbeg + chunk * SKD_CHUNK;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int row = 2 * j + lrow;
+            const int nrow = tile * 16 + row < N ? tile * 16 + row : N - 1;
+            const size_t off = (size_t)nrow * K + k0 + (lpos ^ (row & 15)) * 8;
+            __builtin_amdgcn_global_load_lds(DMA_GP(w + off), DMA_LP(st + 2 * j * SKD_CHUNK), 16, 0, 0);
+            if (SWIGLU) __builtin_amdgcn_global_load_lds(DMA_GP(w2 + off), DMA_LP(st + TILE + 2 * j * SKD_CHUNK), 16, 0, 0);
+        }
+    };
+    auto load_x = [&](int set, int item) {
+        const int chunk = item % nchunks;
+#pragma unroll
+        for (int u = 0; u < 8; ++u) a[set][u] = load8(xp + chunk * SKD_CHUNK + 32 * u);
+    };
+    float4_t acc = {0.f, 0.f, 0.f, 0.f}, acc2 = {0.f, 0.f, 0.f, 0.f};
+    auto consume = [&](int set, int item) {
+        const half_t *st = mine + (size_t)(item & 1) * NW * TILE + r * SKD_CHUNK;
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int pch = (4 * u + g) ^ r; // r < 16
+            const half8_t b = load8(st + pch * 8);
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[set][u], b, acc, 0, 0, 0);
+            if (SWIGLU) {
+                const half8_t b2 = load8(st + TILE + pch * 8);
+                acc2 = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[set][u], b2, acc2, 0, 0, 0);
+            }
+        }
+    };
+    // end of a tile: k-slices of the waves are added in wave order, then the epilogue
+    auto flush = [&](int item) {
+        const int n0 = (blockIdx.x + (item / nchunks) * gridDim.x) * 16;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            red[0][wave][lane][i] = acc[i];
+            if (SWIGLU) red[NW - 1][wave][lane][i] = acc2[i];
+            acc[i] = 0.f;
+            acc2[i] = 0.f;
+        }
+        __syncthreads();
+        if (wave == 0) {
+            const int n = n0 + lane % 16;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int m = 4 * (lane / 16) + i;
+                float s = 0.f, s2 = 0.f;
+#pragma unroll
+                for (int wv = 0; wv < WAVES; ++wv) {
+                    s += red[0][wv][lane][i];
+                    if (SWIGLU) s2 += red[NW - 1][wv][lane][i];
+                }
+                if (m < T && n < N) {
+                    if (SWIGLU) out[(size_t)m * ldo + n] = (half_t)(silu_g(s) * s2);
+                    else out[(size_t)m * ldo + n] = finish(s, res ? res + (size_t)m * ldr + n : nullptr);
+                }
+            }
+        }
+        __syncthreads();
+    };
+    // one step of the pipeline with compile-time register set SET (= parity of the item)
+    auto step = [&](auto set_tag, int item) {
+        constexpr int SET = decltype(set_tag)::value;
+        if (item + 1 < n_items) {
+            issue(item + 1);
+            load_x(SET ^ 1, item + 1);
+            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(VM_PER_CHUNK) : "memory");
+        } else {
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        }
+        consume(SET, item);
+        // the reads of this stage must have returned before the item after next overwrites it
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        if (item % nchunks == nchunks - 1) flush(item);
+    };
+    if (n_items > 0) {
+        issue(0);
+        load_x(0, 0);
+    }
+    for (int item = 0; item < n_items; item += 2) {
+        step(std::integral_constant<int, 0>{}, item);
+        if (item + 1 < n_items) step(std::integral_constant<int, 1>{}, item + 1);
+    }
+}
+
+template <bool SWIGLU, int WAVES>
+static int skinny_dma_launch(const half_t *x, int ldx, const half_t *w, const half_t *w2, const half_t *res, int ldr,
+                             half_t *out, int ldo, int T, int N, int K, hipStream_t s) {
+    const size_t smem = sizeof(half_t) * (size_t)WAVES * 2 * (SWIGLU ? 2 : 1) * 16 * SKD_CHUNK;
+    auto kern = skinny_dma_kernel<SWIGLU, WAVES>;
+    static bool attr_set = false;
+    if (!attr_set) {
+        LLM_HIP_CHECK(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+        attr_set = true;
+    }
+    // the LDS tiles allow one workgroup per CU: as many workgroups as CUs, each walking over column tiles
+    static int cus = 0;
+    if (cus == 0) {
+        int dev = 0;
+        LLM_HIP_CHECK(hipGetDevice(&dev));
+        LLM_HIP_CHECK(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+    }
+    const int tiles = (N + 15) / 16;
+    kern<<<dim3(tiles < cus ? tiles : cus), dim3(WAVES * 64), smem, s>>>(x, ldx, w, w2, res, ldr, out, ldo, T, N, K);
+    LLM_LAUNCH_CHECK("skinny_dma_kernel");
+    return LLM_OK;
 }
 
 // ---------------------------------------------------------------------------
@@ -323,8 +478,6 @@ static int gemm_launch(const half_t *x, int ldx, const half_t *w, const half_t *
 // chunk (l%4) ^ ((row>>2)&3) of its row, so that the 16 lanes an LDS read serves per cycle (16 rows,
 // same logical chunk) fall into 16 different 16-byte bank groups.
 #define DMA_BK 32
-#define DMA_GP(p) ((const __attribute__((address_space(1))) void *)(p))
-#define DMA_LP(p) ((__attribute__((address_space(3))) void *)(p))
 
 template <int N> __device__ __forceinline__ void dma_wait_barrier() {
     // vmcnt(N): all but the newest N of this wave's loads have landed; then the workgroup barrier.
@@ -638,6 +791,8 @@ int llm_linear(const uint16_t *x, int ldx, const uint16_t *w, const uint16_t *re
     const half_t *xp = (const half_t *)x, *wp = (const half_t *)w, *rp = (const half_t *)residual;
     half_t *op = (half_t *)out;
     if (T == 1) return gemv_launch(xp, nullptr, 0.0, wp, rp, op, N, K, s);
+    if (T <= 16 && K % (8 * SKD_CHUNK) == 0 && aligned16(xp) && ldx % 8 == 0)
+        return skinny_dma_launch<false, 8>(xp, ldx, wp, nullptr, rp, ldr, op, ldo, T, N, K, s);
     if (T <= 16 && K % (SK_WAVES * 32) == 0) {
         skinny_kernel<false><<<dim3((N + 15) / 16), dim3(SK_WAVES * 64), 0, s>>>(xp, ldx, wp, nullptr, rp, ldr, op,
                                                                                ldo, T, N, K);
@@ -678,6 +833,8 @@ int llm_linear_swiglu(const uint16_t *x, int ldx, const uint16_t *wgate, const u
     const half_t *xp = (const half_t *)x, *gp = (const half_t *)wgate, *up = (const half_t *)wup;
     half_t *op = (half_t *)out;
     if (T == 1) return gemv_swiglu_launch(xp, nullptr, 0.0, gp, up, op, N, K, s);
+    if (T <= 16 && K % (4 * SKD_CHUNK) == 0)
+        return skinny_dma_launch<true, 4>(xp, ldx, gp, up, nullptr, 0, op, ldo, T, N, K, s);
     if (T <= 16 && K % (SK_WAVES * 32) == 0) {
         skinny_kernel<true><<<dim3((N + 15) / 16), dim3(SK_WAVES * 64), 0, s>>>(xp, ldx, gp, up, nullptr, 0, op, ldo,
                                                                               T, N, K);
