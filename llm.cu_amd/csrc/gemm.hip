@@ -120,133 +120,188 @@ __global__ __launch_bounds__(SK_WAVES * 64) void skinny_kernel(const half_t *__r
 // ---------------------------------------------------------------------------
 // The kernel above reads, per load instruction, 64 bytes from each of 16 weight rows.  Here every wave
 // instruction moves 512 contiguous bytes of two rows straight into the wave's own LDS tile
-// (global_load_lds), i.e. the DRAM pattern of the GEMV, and the MFMA fragments are read back from LDS.
+// (buffer_load ... lds), i.e. the DRAM pattern of the GEMV, and the MFMA fragments are read back from LDS.
 // Same work split: workgroup = 16 output columns, WAVES wavefronts each own a k-slice and process it in
-// chunks of 256; two chunks per wave are in LDS, one being consumed while the next lands (no workgroup
-// barrier: the tiles are private to the wave).  Lane l of an instruction fetches 16-byte chunk
+// chunks of 256; D + 1 chunks per wave are in LDS, one being consumed while the next ones land (no
+// workgroup barrier: the tiles are private to the wave).  Measured at the 8B shapes, a ring of two tiles
+// with four waves is as fast as or faster than deeper rings or more waves.  Lane l of an instruction fetches 16-byte chunk
 // (l%32) ^ (row&15) of its row so that the 16 rows a fragment read touches per cycle sit in 16
 // different bank groups.
 #define SKD_CHUNK 256
 
-template <bool SWIGLU, int WAVES>
-__global__ __launch_bounds__(WAVES * 64) void skinny_dma_kernel(const half_t *__restrict__ x, int ldx,
-                                                                const half_t *__restrict__ w,
-                                                                const half_t *__restrict__ w2, const half_t *res,
-                                                                int ldr, half_t *out, int ldo, int T, int N, int K) {
+template <int N> __device__ __forceinline__ void skd_wait_vm() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
+
+// D = chunks in flight ahead of the one being consumed (LDS ring of D + 1 tiles per wave). N % 16 == 0.
+// XLDS: the x chunk travels like a weight tile (row-contiguous loads into LDS, fragments read back from
+// there) instead of straight into registers, where one load instruction touches 16 rows of 64 bytes.
+template <bool SWIGLU, int WAVES, int D, bool XLDS>
+__global__ __launch_bounds__(WAVES * 64, 1) void skinny_dma_kernel(const half_t *__restrict__ x, int ldx,
+                                                                   const half_t *__restrict__ w,
+                                                                   const half_t *__restrict__ w2, const half_t *res,
+                                                                   int ldr, half_t *out, int ldo, int T, int N, int K) {
     constexpr int NW = SWIGLU ? 2 : 1;
+    constexpr int NS = D + 1;                         // ring slots = register sets
     constexpr int TILE = 16 * SKD_CHUNK;              // halves per weight tile (8 KB)
-    constexpr int VM_PER_CHUNK = 8 * NW + 8;          // load instructions a chunk issues (weights + x)
-    extern __shared__ __attribute__((aligned(16))) half_t sk_lds[]; // [WAVES][2 stages][NW][TILE]
-    __shared__ float red[NW][WAVES][64][4];
-    const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
+    constexpr int VM = 8 * NW + 8;                    // load instructions a chunk issues (weights + x)
+    static_assert(D >= 1 && D <= 3 && D * VM <= 63, "vmcnt counts at most 63 outstanding loads");
+    constexpr int SLOT = (NW + (XLDS ? 1 : 0)) * TILE; // halves per ring slot
+    extern __shared__ __attribute__((aligned(16))) half_t sk_lds[]; // [WAVES][NS][SLOT]
+    __shared__ float red[2][NW][WAVES][64][4];
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64), lane = threadIdx.x % 64;
     const int r = lane % 16, g = lane / 16;
     const int mrow = r < T ? r : T - 1;
     const int kslice = K / WAVES; // multiple of SKD_CHUNK
     const int kbeg = wave * kslice;
     const int nchunks = kslice / SKD_CHUNK;
-    half_t *mine = sk_lds + (size_t)wave * 2 * NW * TILE;
+    half_t *mine = sk_lds + (size_t)wave * NS * SLOT;
     // The workgroup walks over column tiles blockIdx.x, blockIdx.x + gridDim.x, ...; its waves see one
-    // flat sequence of (tile, chunk) items, so the first chunk of the next tile is already on its way
-    // while the last chunk of the current one is consumed and reduced.
-    const int n_tiles = (N + 15) / 16;
-    const int my_tiles = ((int)blockIdx.x < n_tiles) ? (n_tiles - 1 - (int)blockIdx.x) / (int)gridDim.x + 1 : 0;
-    const int n_items = my_tiles * nchunks;
+    // flat sequence of (tile, chunk) items, so the first chunks of the next tile are already on their
+    // way while the last chunk of the current one is consumed and reduced.
+    const int n_tiles = N / 16;
 
-    const int lrow = lane / 32, lpos = lane % 32;
-    const half_t *xp = x + (size_t)mrow * ldx + kbeg + 8 * g;
-    half8_t a[2][8];
-    auto issue = [&](int item) {
-        const int tile = blockIdx.x + (item / nchunks) * gridDim.x, chunk = item % nchunks;
-        half_t *st = mine + (size_t)(item & 1) * NW * TILE;
-        const int k0 = kbeg + chunk * SKD_CHUNK;
+    // element offset of this lane's 16 bytes inside a tile, per load instruction (two rows each)
+    uint32_t lane_off[8], lane_off_x[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const int row = 2 * j + lane / 32;
+        const uint32_t swz = (uint32_t)(((lane % 32) ^ (row & 15)) * 8);
+        lane_off[j] = (uint32_t)row * (uint32_t)K + swz;
+        if (XLDS) lane_off_x[j] = (uint32_t)(row < T ? row : T - 1) * (uint32_t)ldx + swz;
+    }
+    const half_t *xrow = x + (size_t)mrow * ldx + kbeg + 8 * g;
+    half8_t a[XLDS ? 1 : NS][8];
+    // Loads are issued at every ring step, also past the last item: there all lanes fetch the first 16
+    // bytes of the weights (one cache line, never consumed). The number of loads in flight is then the
+    // same at every step, so one constant vmcnt marks the arrival of the item about to be consumed.
+    // The weights go to LDS through buffer loads: with the flat-encoded LDS loads in flight the compiler
+    // turns every wait for the x registers into a wait for all loads, which empties the ring.
+    const int w_bytes = N * K * (int)sizeof(half_t); // < 2^31, checked by the launcher
+    const __amdgpu_buffer_rsrc_t rs_w = __builtin_amdgcn_make_buffer_rsrc((void *)w, 0, w_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rs_w2 = __builtin_amdgcn_make_buffer_rsrc((void *)(SWIGLU ? w2 : w), 0, w_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rs_x =
+        __builtin_amdgcn_make_buffer_rsrc((void *)x, 0, ((T - 1) * ldx + K) * (int)sizeof(half_t), 0x00020000);
+    int c_tile = blockIdx.x, c_chunk = 0; // issue cursor
+    auto issue = [&](int slot) {
+        const bool live = c_tile < n_tiles;
+        const uint32_t keep = live ? 0xffffffffu : 0u;
+        const uint32_t base = live ? ((uint32_t)c_tile * 16u * (uint32_t)K + kbeg + c_chunk * SKD_CHUNK) * 2u : 0u;
+        half_t *st = mine + (size_t)slot * SLOT;
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
-            const int row = 2 * j + lrow;
-            const int nrow = tile * 16 + row < N ? tile * 16 + row : N - 1;
-            const size_t off = (size_t)nrow * K + k0 + (lpos ^ (row & 15)) * 8;
-            __builtin_amdgcn_global_load_lds(DMA_GP(w + off), DMA_LP(st + 2 * j * SKD_CHUNK), 16, 0, 0);
-            if (SWIGLU) __builtin_amdgcn_global_load_lds(DMA_GP(w2 + off), DMA_LP(st + TILE + 2 * j * SKD_CHUNK), 16, 0, 0);
+            const uint32_t off = (lane_off[j] & keep) * 2u;
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_w, DMA_LP(st + 2 * j * SKD_CHUNK), 16, off, base, 0, 0);
+            if (SWIGLU)
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_w2, DMA_LP(st + TILE + 2 * j * SKD_CHUNK), 16, off, base, 0, 0);
+        }
+        // x is always read at the cursor's chunk (valid also past the last item); the empty asm hides the
+        // offset from the optimiser, which would otherwise replace a repeated load by a register copy
+        // and change the number of loads in flight
+        int xoff = c_chunk * SKD_CHUNK;
+        if (XLDS) {
+            const uint32_t xbase = (uint32_t)(kbeg + xoff) * 2u;
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_x, DMA_LP(st + NW * TILE + 2 * j * SKD_CHUNK), 16,
+                                                         lane_off_x[j] * 2u, xbase, 0, 0);
+        } else {
+            asm volatile("" : "+s"(xoff));
+            const half_t *xs = xrow + xoff;
+#pragma unroll
+            for (int u = 0; u < 8; ++u) a[slot][u] = load8(xs + 32 * u);
+        }
+        if (++c_chunk == nchunks) {
+            c_chunk = 0;
+            c_tile += gridDim.x;
         }
     };
-    auto load_x = [&](int set, int item) {
-        const int chunk = item % nchunks;
-#pragma unroll
-        for (int u = 0; u < 8; ++u) a[set][u] = load8(xp + chunk * SKD_CHUNK + 32 * u);
-    };
     float4_t acc = {0.f, 0.f, 0.f, 0.f}, acc2 = {0.f, 0.f, 0.f, 0.f};
-    auto consume = [&](int set, int item) {
-        const half_t *st = mine + (size_t)(item & 1) * NW * TILE + r * SKD_CHUNK;
+    auto consume = [&](int slot) {
+        const half_t *st = mine + (size_t)slot * SLOT + r * SKD_CHUNK;
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
             const int pch = (4 * u + g) ^ r; // r < 16
             const half8_t b = load8(st + pch * 8);
-            acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[set][u], b, acc, 0, 0, 0);
+            const half8_t af = XLDS ? load8(st + NW * TILE + pch * 8) : a[XLDS ? 0 : slot][u];
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(af, b, acc, 0, 0, 0);
             if (SWIGLU) {
                 const half8_t b2 = load8(st + TILE + pch * 8);
-                acc2 = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[set][u], b2, acc2, 0, 0, 0);
+                acc2 = __builtin_amdgcn_mfma_f32_16x16x32_f16(af, b2, acc2, 0, 0, 0);
             }
         }
     };
-    // end of a tile: k-slices of the waves are added in wave order, then the epilogue
-    auto flush = [&](int item) {
-        const int n0 = (blockIdx.x + (item / nchunks) * gridDim.x) * 16;
+    // End of a tile: the k-slices of the waves are added in wave order by one wave, which then runs the
+    // epilogue. The partial sums alternate between two buffers, so one barrier per tile is enough (a wave
+    // reaches the buffer of tile t again only behind the barrier of tile t + 1), and the epilogue wave
+    // rotates, so the wait for the residual values is not always the same wave's.
+    int u_tile = blockIdx.x, u_chunk = 0, flip = 0, ep_wave = 0; // consume cursor
+    auto flush = [&]() {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            red[0][wave][lane][i] = acc[i];
-            if (SWIGLU) red[NW - 1][wave][lane][i] = acc2[i];
+            red[flip][0][wave][lane][i] = acc[i];
+            if (SWIGLU) red[flip][NW - 1][wave][lane][i] = acc2[i];
             acc[i] = 0.f;
             acc2[i] = 0.f;
         }
-        __syncthreads();
-        if (wave == 0) {
-            const int n = n0 + lane % 16;
+        // workgroup barrier without a wait on the loads in flight
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        if (wave == ep_wave) {
+            const int n = u_tile * 16 + lane % 16;
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const int m = 4 * (lane / 16) + i;
                 float s = 0.f, s2 = 0.f;
 #pragma unroll
                 for (int wv = 0; wv < WAVES; ++wv) {
-                    s += red[0][wv][lane][i];
-                    if (SWIGLU) s2 += red[NW - 1][wv][lane][i];
+                    s += red[flip][0][wv][lane][i];
+                    if (SWIGLU) s2 += red[flip][NW - 1][wv][lane][i];
                 }
-                if (m < T && n < N) {
+                if (m < T) {
                     if (SWIGLU) out[(size_t)m * ldo + n] = (half_t)(silu_g(s) * s2);
                     else out[(size_t)m * ldo + n] = finish(s, res ? res + (size_t)m * ldr + n : nullptr);
                 }
             }
         }
-        __syncthreads();
+        flip ^= 1;
+        ep_wave = ep_wave + 1 == WAVES ? 0 : ep_wave + 1;
     };
-    // one step of the pipeline with compile-time register set SET (= parity of the item)
-    auto step = [&](auto set_tag, int item) {
-        constexpr int SET = decltype(set_tag)::value;
-        if (item + 1 < n_items) {
-            issue(item + 1);
-            load_x(SET ^ 1, item + 1);
-            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(VM_PER_CHUNK) : "memory");
-        } else {
-            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    // one step with compile-time ring slot SLOT: refill the slot freed by the previous step, wait for
+    // this item's loads, consume
+    auto step = [&](auto slot_tag) {
+        constexpr int SLOT = decltype(slot_tag)::value;
+        issue((SLOT + D) % NS);
+        skd_wait_vm<D * VM>();
+        if (u_tile < n_tiles) {
+            consume(SLOT);
+            // the reads of this slot must have returned before the next step refills it
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            if (++u_chunk == nchunks) {
+                flush();
+                u_chunk = 0;
+                u_tile += gridDim.x;
+            }
         }
-        consume(SET, item);
-        // the reads of this stage must have returned before the item after next overwrites it
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-        if (item % nchunks == nchunks - 1) flush(item);
     };
-    if (n_items > 0) {
-        issue(0);
-        load_x(0, 0);
+#pragma unroll
+    for (int i = 0; i < D; ++i) issue(i);
+    while (u_tile < n_tiles) {
+        step(std::integral_constant<int, 0>{});
+        if (NS > 1) step(std::integral_constant<int, 1 % NS>{});
+        if (NS > 2) step(std::integral_constant<int, 2 % NS>{});
+        if (NS > 3) step(std::integral_constant<int, 3 % NS>{});
     }
-    for (int item = 0; item < n_items; item += 2) {
-        step(std::integral_constant<int, 0>{}, item);
-        if (item + 1 < n_items) step(std::integral_constant<int, 1>{}, item + 1);
-    }
+    skd_wait_vm<0>(); // the filler loads still write into this workgroup's LDS
 }
 
-template <bool SWIGLU, int WAVES>
+// whole 16-column tiles, and byte offsets into the weights that fit the 32-bit buffer addressing
+static bool skd_fits(int N, int K) { return N % 16 == 0 && (size_t)N * K * sizeof(half_t) < ((size_t)1 << 31); }
+
+template <bool SWIGLU, int WAVES, int D, bool XLDS>
 static int skinny_dma_launch(const half_t *x, int ldx, const half_t *w, const half_t *w2, const half_t *res, int ldr,
                              half_t *out, int ldo, int T, int N, int K, hipStream_t s) {
-    const size_t smem = sizeof(half_t) * (size_t)WAVES * 2 * (SWIGLU ? 2 : 1) * 16 * SKD_CHUNK;
-    auto kern = skinny_dma_kernel<SWIGLU, WAVES>;
+    const size_t smem = sizeof(half_t) * (size_t)WAVES * (D + 1) * ((SWIGLU ? 2 : 1) + (XLDS ? 1 : 0)) * 16 * SKD_CHUNK;
+    static_assert(sizeof(half_t) * WAVES * (D + 1) * ((SWIGLU ? 2 : 1) + (XLDS ? 1 : 0)) * 16 * SKD_CHUNK <= 144 * 1024,
+                  "ring does not fit beside the reduction buffers");
+    auto kern = skinny_dma_kernel<SWIGLU, WAVES, D, XLDS>;
     static bool attr_set = false;
     if (!attr_set) {
         LLM_HIP_CHECK(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
@@ -791,8 +846,8 @@ int llm_linear(const uint16_t *x, int ldx, const uint16_t *w, const uint16_t *re
     const half_t *xp = (const half_t *)x, *wp = (const half_t *)w, *rp = (const half_t *)residual;
     half_t *op = (half_t *)out;
     if (T == 1) return gemv_launch(xp, nullptr, 0.0, wp, rp, op, N, K, s);
-    if (T <= 16 && K % (8 * SKD_CHUNK) == 0 && aligned16(xp) && ldx % 8 == 0)
-        return skinny_dma_launch<false, 8>(xp, ldx, wp, nullptr, rp, ldr, op, ldo, T, N, K, s);
+    if (T <= 16 && skd_fits(N, K) && K % (4 * SKD_CHUNK) == 0 && aligned16(xp) && ldx % 8 == 0)
+        return skinny_dma_launch<false, 4, 1, true>(xp, ldx, wp, nullptr, rp, ldr, op, ldo, T, N, K, s);
     if (T <= 16 && K % (SK_WAVES * 32) == 0) {
         skinny_kernel<false><<<dim3((N + 15) / 16), dim3(SK_WAVES * 64), 0, s>>>(xp, ldx, wp, nullptr, rp, ldr, op,
                                                                                ldo, T, N, K);
@@ -833,8 +888,9 @@ int llm_linear_swiglu(const uint16_t *x, int ldx, const uint16_t *wgate, const u
     const half_t *xp = (const half_t *)x, *gp = (const half_t *)wgate, *up = (const half_t *)wup;
     half_t *op = (half_t *)out;
     if (T == 1) return gemv_swiglu_launch(xp, nullptr, 0.0, gp, up, op, N, K, s);
-    if (T <= 16 && K % (4 * SKD_CHUNK) == 0)
-        return skinny_dma_launch<true, 4>(xp, ldx, gp, up, nullptr, 0, op, ldo, T, N, K, s);
+    if (T <= 16 && skd_fits(N, K) && K % (4 * SKD_CHUNK) == 0)
+        // x straight into registers here: with two weight tiles per slot the LDS ring has no room for x
+        return skinny_dma_launch<true, 4, 1, false>(xp, ldx, gp, up, nullptr, 0, op, ldo, T, N, K, s);
     if (T <= 16 && K % (SK_WAVES * 32) == 0) {
         skinny_kernel<true><<<dim3((N + 15) / 16), dim3(SK_WAVES * 64), 0, s>>>(xp, ldx, gp, up, nullptr, 0, op, ldo,
                                                                               T, N, K);
