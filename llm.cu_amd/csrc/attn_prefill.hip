@@ -54,8 +54,11 @@ __global__ __launch_bounds__(G *AP_QT * 64) void attn_prefill_kernel(const half_
     half_t *Vt = smem + 2 * KTILE; // [2][VTILE]
 
     const int n_qt = (T + AP_BQ - 1) / AP_BQ;
-    const int blk = gridDim.x - 1 - blockIdx.x; // longest rows first
-    const int kvh = blockIdx.y;
+    // Workgroups are dispatched in the order of their linear id, x fastest.  KV head on x, row block on
+    // y, longest rows first: the long workgroups of all heads start first and the short ones fill the
+    // tail, and consecutive ids (which go round the XCDs) keep one KV head per XCD and its L2.
+    const int blk = gridDim.y - 1 - blockIdx.y;
+    const int kvh = blockIdx.x;
     const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
     const int head = kvh * G + wave % G;
     int qtile = blk * AP_QT + wave / G;
@@ -116,6 +119,10 @@ __global__ __launch_bounds__(G *AP_QT * 64) void attn_prefill_kernel(const half_
 
     gload(0);
     sstore(0);
+    // All loads issued so far (the query fragments among them) are complete from here on.  Without this
+    // wait the compiler, which cannot tell the first pass of the loop from the others, makes every pass
+    // wait for the query registers with counts that also drain the K/V prefetch issued at its top.
+    __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0)
     __syncthreads();
     for (int kt = 0; kt < n_tiles; ++kt) {
         const int key0 = kt * AP_BKEY;
@@ -217,7 +224,7 @@ static int launch_prefill(const half_t *q, int ldq, const half_t *kc, const half
                           int T, int pos0, int n_kv_heads, int max_pos, hipStream_t s) {
     constexpr int AP_QT = G >= 8 ? 1 : 2; // 32-row query tiles per workgroup (at most 8 wavefronts)
     const int n_qt = (T + AP_BQ - 1) / AP_BQ;
-    dim3 grid((n_qt + AP_QT - 1) / AP_QT, n_kv_heads);
+    dim3 grid(n_kv_heads, (n_qt + AP_QT - 1) / AP_QT);
     const size_t smem = sizeof(half_t) * 2 * ((size_t)AP_BKEY * (HD + 8) + (size_t)HD * (AP_BKEY + 8));
     auto kern = attn_prefill_kernel<HD, G, AP_QT>;
     static bool attr_set = false;
