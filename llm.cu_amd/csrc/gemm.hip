@@ -558,7 +558,6 @@ __global__ __launch_bounds__(WGM * WGN * 64, OCC) void gemm_dma_kernel(const hal
     constexpr int STAGE_HALVES = (BM + BROWS) * DMA_BK;
     constexpr int LPT = (BM + BROWS) / 16 / NWAVES; // load instructions per wave per tile
     constexpr int AHEAD = PREF ? STAGES - 2 : STAGES - 1;
-    static_assert((BM + BROWS) / 16 % NWAVES == 0, "loader split");
     extern __shared__ __attribute__((aligned(16))) half_t lds[];
 
     const int nblk = tiles_m * tiles_n;
@@ -575,36 +574,51 @@ __global__ __launch_bounds__(WGM * WGN * 64, OCC) void gemm_dma_kernel(const hal
     const int tn = (bid % (GROUP_M * tiles_n)) / gsz;
     const int m0 = tm * BM, n0 = tn * BN;
 
-    const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
+    const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid / 64), lane = tid % 64;
     const int wm = wave % WGM, wn = wave / WGM;
     const int kbeg = ws ? blockIdx.y * kper : 0;
 
-    // loader: instruction q of a tile moves 16 rows x 64 B (q < BM/16: A rows, else B rows);
-    // lane -> row lane/4, LDS chunk lane%4 holding global chunk (lane%4) ^ ((row>>2)&3)
+    // loader: instruction q = t * NWAVES + wave of a tile moves 16 rows x 64 B (q < BM/16: A rows, else B
+    // rows); lane -> row lane/4, LDS chunk lane%4 holding global chunk (lane%4) ^ ((row>>2)&3).  Buffer
+    // loads with LDS destination: the per-lane byte offset is fixed, the k offset travels in the scalar
+    // offset, so a tile costs no vector ALU work; and, unlike the flat-encoded LDS loads, they do not make
+    // the compiler turn every LDS wait into lgkmcnt(0).
+    constexpr int TA = BM / 16 / NWAVES, TB1 = BN / 16 / NWAVES; // instructions per wave: A, one B matrix
+    static_assert(BM / 16 % NWAVES == 0 && BN / 16 % NWAVES == 0 && TA + NB * TB1 == LPT, "loader split");
     const int lrow = lane / 4, lchunk = (lane & 3) ^ ((lane >> 4) & 3);
-    const half_t *gp[LPT];
+    const __amdgpu_buffer_rsrc_t rs_x =
+        __builtin_amdgcn_make_buffer_rsrc((void *)x, 0, ((T - 1) * ldx + K) * (int)sizeof(half_t), 0x00020000);
+    const __amdgpu_buffer_rsrc_t rs_w = __builtin_amdgcn_make_buffer_rsrc((void *)w, 0, N * K * (int)sizeof(half_t), 0x00020000);
+    const __amdgpu_buffer_rsrc_t rs_w2 =
+        __builtin_amdgcn_make_buffer_rsrc((void *)(NB == 2 ? w2 : w), 0, N * K * (int)sizeof(half_t), 0x00020000);
+    // fixed bound: an array whose size depends on the template arguments, captured by the lambdas below, makes
+    // this compiler drop the host stub of the kernel without a diagnostic
+    static_assert(LPT <= 16, "goff");
+    uint32_t goff[16];
 #pragma unroll
     for (int t = 0; t < LPT; ++t) {
         const int q = wave + t * NWAVES;
-        if (q < BM / 16) {
+        if (t < TA) {
             int ar = m0 + q * 16 + lrow;
             ar = ar < T ? ar : T - 1;
-            gp[t] = x + (size_t)ar * ldx + kbeg + lchunk * 8;
+            goff[t] = ((uint32_t)ar * (uint32_t)ldx + kbeg + lchunk * 8) * 2u;
         } else {
-            int brl = (q - BM / 16) * 16 + lrow;
-            const half_t *wb = w;
-            if (NB == 2 && brl >= BN) { wb = w2; brl -= BN; }
-            int br = n0 + brl;
+            int br = n0 + (q - BM / 16) * 16 + lrow - (t >= TA + TB1 ? BN : 0);
             br = br < N ? br : N - 1;
-            gp[t] = wb + (size_t)br * K + kbeg + lchunk * 8;
+            goff[t] = ((uint32_t)br * (uint32_t)K + kbeg + lchunk * 8) * 2u;
         }
     }
-    auto issue = [&](int kt) {
+    auto issue_one = [&](int kt, int t) {
         half_t *st = lds + (kt % STAGES) * STAGE_HALVES;
-        const int k0 = kt * DMA_BK;
+        const uint32_t k0 = (uint32_t)kt * DMA_BK * 2u;
+        auto dst = DMA_LP(st + (wave + t * NWAVES) * 16 * DMA_BK);
+        if (t < TA) __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_x, dst, 16, goff[t], k0, 0, 0);
+        else if (t < TA + TB1) __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_w, dst, 16, goff[t], k0, 0, 0);
+        else __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_w2, dst, 16, goff[t], k0, 0, 0);
+    };
+    auto issue = [&](int kt) {
 #pragma unroll
-        for (int t = 0; t < LPT; ++t)
-            __builtin_amdgcn_global_load_lds(DMA_GP(gp[t] + k0), DMA_LP(st + (wave + t * NWAVES) * 16 * DMA_BK), 16, 0, 0);
+        for (int t = 0; t < LPT; ++t) issue_one(kt, t);
     };
 
     const int frow = lane % 32, sw = (frow >> 2) & 3;
@@ -648,25 +662,56 @@ __global__ __launch_bounds__(WGM * WGN * 64, OCC) void gemm_dma_kernel(const hal
         if (t < nk) issue(t);
     // tiles issued so far: min(nk, AHEAD + PREF).  Loop invariant at the top of iteration kt: tiles up to
     // kt + (PREF ? 1 : 0) have landed for every wave, tiles up to kt + AHEAD - (PREF ? 0 : 1) ... are in flight.
-    if (PREF) {
+    if constexpr (PREF) {
         const int beyond = (nk < AHEAD + 1 ? nk : AHEAD + 1) - 2;
         if (beyond >= 2) dma_wait_barrier<2 * LPT>();
         else if (beyond == 1) dma_wait_barrier<LPT>();
         else dma_wait_barrier<0>();
         lfrag(0, 0, 0);
-        for (int kt = 0; kt < nk; ++kt) {
-            __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0): fragments prefetched last iteration are in
-            if (kt + AHEAD + 1 < nk) issue(kt + AHEAD + 1);
-            lfrag(1, kt, 1);
-            __builtin_amdgcn_sched_barrier(0);
-            mma(0);
-            __builtin_amdgcn_sched_barrier(0);
-            if (kt + 1 < nk) lfrag(0, kt + 1, 0);
-            __builtin_amdgcn_sched_barrier(0);
-            mma(1);
-            __builtin_amdgcn_sched_barrier(0);
-            const int last = kt + AHEAD + 1 < nk - 1 ? kt + AHEAD + 1 : nk - 1;
-            const int beyond2 = last - (kt + 2);
+        // One pass = one BK step: 2 x 16 MFMAs on fragment sets 0 and 1.  Set 1 of this step and set 0 of the
+        // next are read from LDS while the MFMAs run (set 0 of a step past the end reads a stale stage and is
+        // never used: no branch inside the pass), the loads of the step AHEAD + 1 further on are issued first.
+        // The instruction order of a pass is written out and pinned (a scheduling fence after every MFMA):
+        // behind MFMA i of the first block one LDS read of set 1, then one tile load; behind MFMA i of the
+        // second block one LDS read of set 0 of the next step.  Left alone the scheduler packs the reads right
+        // in front of their MFMAs to save registers and exposes the LDS latency.
+        constexpr int MM = 4 * FM, RD = FM + 4;
+        static_assert(RD + LPT <= MM, "more loads than MFMAs to hide them behind");
+        auto one_read = [&](int set, int kt, int ks, int r) {
+            const half_t *st = lds + (kt % STAGES) * STAGE_HALVES;
+            if (r < FM) af[set][r] = load8(st + a_off[ks] + r * 32 * DMA_BK);
+            else {
+                const int f = r - FM;
+                const int roff = NB == 1 ? f * 32 : (f / 2) * BN + (f % 2) * 32;
+                bf[set][f] = load8(st + b_off[ks] + roff * DMA_BK);
+            }
+        };
+        auto pass = [&](int kt, auto with_issue) {
+#pragma unroll
+            for (int i = 0; i < MM; ++i) {
+                acc[i / FM][i % FM] =
+                    __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[0][i / FM], af[0][i % FM], acc[i / FM][i % FM], 0, 0, 0);
+                if (i < RD) one_read(1, kt, 1, i);
+                else if (decltype(with_issue)::value && i - RD < LPT) issue_one(kt + AHEAD + 1, i - RD);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+#pragma unroll
+            for (int i = 0; i < MM; ++i) {
+                acc[i / FM][i % FM] =
+                    __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[1][i / FM], af[1][i % FM], acc[i / FM][i % FM], 0, 0, 0);
+                if (i < RD) one_read(0, kt + 1, 0, i);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        };
+        int kt = 0;
+        for (; kt + AHEAD + 1 < nk; ++kt) {
+            pass(kt, std::true_type{});
+            // tile kt + 2 must have landed; issued after it: tiles kt + 3 .. kt + AHEAD + 1
+            dma_wait_barrier<(AHEAD - 1) * LPT>();
+        }
+        for (; kt < nk; ++kt) {
+            pass(kt, std::false_type{});
+            const int beyond2 = nk - 1 - (kt + 2); // tiles in flight after kt + 2
             if (AHEAD >= 3 && beyond2 >= 2) dma_wait_barrier<2 * LPT>();
             else if (beyond2 >= 1) dma_wait_barrier<LPT>();
             else dma_wait_barrier<0>();
@@ -830,8 +875,11 @@ static int check_linear(const void *x, int ldx, const void *w, const void *out, 
 }
 
 // the direct-to-LDS kernels store (and read the residual) four halves at a time
-static bool dma_ok(const half_t *out, int ldo, const half_t *res, int ldr) {
-    return ((uintptr_t)out & 7u) == 0 && ldo % 4 == 0 && (!res || (((uintptr_t)res & 7u) == 0 && ldr % 4 == 0));
+// the tiles are fetched with 32-bit byte offsets into x and w
+static bool dma_ok(const half_t *out, int ldo, const half_t *res, int ldr, int T, int ldx, int N, int K) {
+    const size_t lim = (size_t)1 << 31;
+    return ((uintptr_t)out & 7u) == 0 && ldo % 4 == 0 && (!res || (((uintptr_t)res & 7u) == 0 && ldr % 4 == 0)) &&
+           (size_t)T * ldx * sizeof(half_t) < lim && (size_t)N * K * sizeof(half_t) < lim;
 }
 
 extern "C" {
@@ -854,7 +902,7 @@ int llm_linear(const uint16_t *x, int ldx, const uint16_t *w, const uint16_t *re
         LLM_LAUNCH_CHECK("skinny_kernel");
         return LLM_OK;
     }
-    if (!dma_ok(op, ldo, rp, ldr) || N < 128) {
+    if (!dma_ok(op, ldo, rp, ldr, T, ldx, N, K) || N < 128) {
         if (T <= 64 || N < 256) return gemm_launch<64, 64, 2, 2, 1>(xp, ldx, wp, nullptr, rp, ldr, op, ldo, T, N, K, s);
         return gemm_launch<128, 128, 2, 2, 1>(xp, ldx, wp, nullptr, rp, ldr, op, ldo, T, N, K, s);
     }
@@ -864,10 +912,11 @@ int llm_linear(const uint16_t *x, int ldx, const uint16_t *w, const uint16_t *re
         return gemm_dma_launch<1, 2, 1, 4, false, 2>(xp, ldx, wp, nullptr, rp, ldr, op, ldo, T, N, K,
                                                      pick_splits(tiles, T, N, K), s);
     }
-    // few tiles, short K: two independent 4-wave workgroups per CU hide each other's prologue and
-    // epilogue; otherwise the 8-wave 256 x 256 tile with the deeper pipeline wins
+    // Measured at the 8B shapes: once the 256 x 256 tiles cover about three quarters of the CUs the
+    // 4-wave tile below with its pinned, interleaved pipeline wins; with fewer tiles the 256 x 128 tile,
+    // two workgroups per CU and a k split where that fills the chip.
     const long tiles = (long)((T + 255) / 256) * ((N + 255) / 256);
-    if (T <= 1024 || (tiles <= 512 && K <= 4096)) {
+    if (tiles < 192) {
         const long t4 = (long)((T + 255) / 256) * ((N + 127) / 128);
         return gemm_dma_launch<1, 4, 1, 3, false, 2>(xp, ldx, wp, nullptr, rp, ldr, op, ldo, T, N, K,
                                                      pick_splits(t4, T, N, K), s);
@@ -897,7 +946,7 @@ int llm_linear_swiglu(const uint16_t *x, int ldx, const uint16_t *wgate, const u
         LLM_LAUNCH_CHECK("skinny_kernel<swiglu>");
         return LLM_OK;
     }
-    if (!dma_ok(op, ldo, nullptr, 0) || N < 64) {
+    if (!dma_ok(op, ldo, nullptr, 0, T, ldx, N, K) || N < 64) {
         if (T <= 64 || N < 256) return gemm_launch<64, 64, 2, 2, 2>(xp, ldx, gp, up, nullptr, 0, op, ldo, T, N, K, s);
         return gemm_launch<128, 64, 2, 2, 2>(xp, ldx, gp, up, nullptr, 0, op, ldo, T, N, K, s);
     }
@@ -905,7 +954,8 @@ int llm_linear_swiglu(const uint16_t *x, int ldx, const uint16_t *wgate, const u
     if (T <= 128)
         return gemm_dma_launch<2, 2, 1, 4, false, 2>(xp, ldx, gp, up, nullptr, 0, op, ldo, T, N, K,
                                                      pick_splits(2 * (long)((N + 63) / 64), T, N, K, 2), s);
-    if (T <= 1024) return gemm_dma_launch<2, 4, 1, 3, false, 2>(xp, ldx, gp, up, nullptr, 0, op, ldo, T, N, K, 1, s);
+    if ((long)((T + 255) / 256) * ((N + 127) / 128) < 192)
+        return gemm_dma_launch<2, 4, 1, 3, false, 2>(xp, ldx, gp, up, nullptr, 0, op, ldo, T, N, K, 1, s);
     return gemm_dma_launch<2, 2, 2, 4, true, 1, 4>(xp, ldx, gp, up, nullptr, 0, op, ldo, T, N, K, 1, s);
 }
 
