@@ -24,6 +24,7 @@
 // P in fp32; the difference is below the fp16 rounding of the output).
 #include <cfloat>
 #include <cmath>
+#include <type_traits>
 
 #include "common.hpp"
 
@@ -90,12 +91,14 @@ __global__ __launch_bounds__(G *AP_QT * 64) void attn_prefill_kernel(const half_
     const int pm = (n & ~0xC) | ((n & 8) >> 1) | ((n & 4) << 1); // pi(n)
 
     half8_t rk[KL], rv[VL];
-    auto gload = [&](int key0) {
+    auto gload_k = [&](int key0) {
 #pragma unroll
         for (int i = 0; i < KL; ++i) {
             const int c = tid + i * THREADS;
             if (KCH % THREADS == 0 || c < KCH) rk[i] = load8(kbase + (size_t)(key0 + c / (HD / 8)) * HD + (c % (HD / 8)) * 8);
         }
+    };
+    auto gload_v = [&](int key0) {
 #pragma unroll
         for (int i = 0; i < VL; ++i) {
             const int c = tid + i * THREADS;
@@ -103,12 +106,14 @@ __global__ __launch_bounds__(G *AP_QT * 64) void attn_prefill_kernel(const half_
                 rv[i] = load8(vbase + (size_t)(c / (AP_BKEY / 8)) * max_pos + key0 + (c % (AP_BKEY / 8)) * 8);
         }
     };
-    auto sstore = [&](int buf) {
+    auto sstore_k = [&](int buf) {
 #pragma unroll
         for (int i = 0; i < KL; ++i) {
             const int c = tid + i * THREADS;
             if (KCH % THREADS == 0 || c < KCH) store8(Ks + buf * KTILE + (c / (HD / 8)) * KLD + (c % (HD / 8)) * 8, rk[i]);
         }
+    };
+    auto sstore_v = [&](int buf) {
 #pragma unroll
         for (int i = 0; i < VL; ++i) {
             const int c = tid + i * THREADS;
@@ -117,90 +122,193 @@ __global__ __launch_bounds__(G *AP_QT * 64) void attn_prefill_kernel(const half_
         }
     };
 
-    gload(0);
-    sstore(0);
-    // All loads issued so far (the query fragments among them) are complete from here on.  Without this
-    // wait the compiler, which cannot tell the first pass of the loop from the others, makes every pass
-    // wait for the query registers with counts that also drain the K/V prefetch issued at its top.
-    __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0)
-    __syncthreads();
-    for (int kt = 0; kt < n_tiles; ++kt) {
-        const int key0 = kt * AP_BKEY;
-        const int buf = kt & 1;
-        if (kt + 1 < n_tiles) gload(key0 + AP_BKEY);
-        if (live && key0 <= my_last) {
-            const half_t *ks = Ks + buf * KTILE, *vt = Vt + buf * VTILE;
-            // S^T for the two 32-key halves of the tile
-            float16_t st[2];
+    // The two matrix products of a tile, with pinned instruction order (a scheduling fence after every
+    // MFMA): accumulators alternate, so no MFMA waits for the one before it, and the LDS fragment of MFMA
+    // i + LA is read behind MFMA i.  Left alone the scheduler reads each fragment right in front of its
+    // MFMA and both wavefronts of a SIMD sit out the LDS latency together.
+    constexpr int NQ = 2 * DS, NP = 4 * DT, LA = 4; // MFMAs per product; read-ahead
+    auto kfrag = [&](const half_t *ks, int i) { return load8(ks + (32 * (i % 2) + pm) * KLD + 8 * hb + 16 * (i / 2)); };
+    auto vfrag = [&](const half_t *vt, int i) { return load8(vt + (32 * (i % DT) + n) * VLD + 16 * (i / DT) + 8 * hb); };
+    // lanes l and l ^ 32 hold the two halves of a query's keys
+    auto xhalf = [&](float x, float &lo, float &hi) {
+        auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+        lo = __uint_as_float(r[0]);
+        hi = __uint_as_float(r[1]);
+    };
+
+    // Softmax of one tile in slices, so that it can run between the MFMAs of the next tile's first product.
+    // The state of the tile in flight lives in these variables; slice i of NQ:
+    //   [0, NQ/4)   running max over the 32 raw scores of the lane
+    //   NQ/4        other half of the keys; new running max m_new, rescale factor alpha
+    //   [NQ/2, NQ)  p = 2^(s*c2 - m_new), partial row sum
+    // sm_finish adds the row sum into l_run and rescales O^T if some lane's max moved.  The softmax runs in
+    // base 2: with c2 = log2(e)/sqrt(hd), p is one fma and one v_exp_f32 per score.
+    float sm_mx = -FLT_MAX, sm_new = 0.f, sm_alpha = 1.f, sm_sum = 0.f;
+    auto sm_slice = [&](float16_t (&st)[2], int i) {
+        constexpr int PM = 128 / NQ, PE = 64 / NQ; // scores per max slice / per exp slice
+        if (i < NQ / 4) {
+            if (i == 0) sm_mx = -FLT_MAX;
 #pragma unroll
-            for (int kh = 0; kh < 2; ++kh) {
-#pragma unroll
-                for (int e = 0; e < 16; ++e) st[kh][e] = 0.f;
-                const half_t *kr = ks + (32 * kh + pm) * KLD + 8 * hb;
-#pragma unroll
-                for (int s = 0; s < DS; ++s)
-                    st[kh] = __builtin_amdgcn_mfma_f32_32x32x16_f16(load8(kr + 16 * s), qf[s], st[kh], 0, 0, 0);
+            for (int j = 0; j < PM; ++j) {
+                const int e = i * PM + j;
+                sm_mx = fmaxf(sm_mx, st[e / 16][e % 16]);
             }
-            // causal mask (only tiles that reach past the first row of this query tile need it) and
-            // running max on the raw scores.  accumulator e of half kh is key
-            // key0 + 32*kh + 16*(e/8) + 8*hb + e%8.  The softmax runs in base 2: with
-            // c = log2(e)/sqrt(hd), p = 2^(s*c - m) is one fma and one v_exp_f32 per score; a masked
-            // score (-FLT_MAX) gives 2^(-huge) = 0 without a select.
-            float mx = -FLT_MAX;
-            if (key0 + AP_BKEY - 1 > pos0 + q0) {
+        }
+        if (i == NQ / 4) {
+            float lo, hi;
+            xhalf(sm_mx, lo, hi);
+            sm_new = fmaxf(m_run, fmaxf(lo, hi) * c2);
+            sm_alpha = __builtin_amdgcn_exp2f(m_run - sm_new);
+            sm_sum = 0.f;
+        }
+        if (i >= NQ / 2) {
 #pragma unroll
-                for (int kh = 0; kh < 2; ++kh)
-#pragma unroll
-                    for (int e = 0; e < 16; ++e) {
-                        const int key = key0 + 32 * kh + 16 * (e / 8) + 8 * hb + (e % 8);
-                        const float sv = key <= qpos ? st[kh][e] : -FLT_MAX;
-                        st[kh][e] = sv;
-                        mx = fmaxf(mx, sv);
-                    }
-            } else {
-#pragma unroll
-                for (int kh = 0; kh < 2; ++kh)
-#pragma unroll
-                    for (int e = 0; e < 16; ++e) mx = fmaxf(mx, st[kh][e]);
+            for (int j = 0; j < PE; ++j) {
+                const int e = (i - NQ / 2) * PE + j;
+                const float p = __builtin_amdgcn_exp2f(fmaf(st[e / 16][e % 16], c2, -sm_new));
+                st[e / 16][e % 16] = p;
+                sm_sum += p;
             }
-            mx = fmaxf(mx, __shfl_xor(mx, 32));
-            const float m_new = fmaxf(m_run, mx * c2);
-            const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
-            float psum = 0.f;
+        }
+    };
+    auto sm_finish = [&]() {
+        float lo, hi;
+        xhalf(sm_sum, lo, hi);
+        l_run = l_run * sm_alpha + (lo + hi);
+        // the running max settles after the first tiles: skip the rescale of O^T when no lane needs it
+        if (__builtin_amdgcn_ballot_w64(sm_new != m_run) != 0) {
+#pragma unroll
+            for (int t = 0; t < DT; ++t)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) o[t][e] *= sm_alpha;
+        }
+        m_run = sm_new;
+    };
+    // causal mask of a tile that reaches past the first row of this query tile: accumulator e of half kh is
+    // key key0 + 32*kh + 16*(e/8) + 8*hb + e%8; a masked score (-FLT_MAX) gives 2^(-huge) = 0
+    auto mask = [&](float16_t (&st)[2], int key0) {
+        if (key0 + AP_BKEY - 1 > pos0 + q0) {
 #pragma unroll
             for (int kh = 0; kh < 2; ++kh)
 #pragma unroll
                 for (int e = 0; e < 16; ++e) {
-                    const float p = __builtin_amdgcn_exp2f(fmaf(st[kh][e], c2, -m_new));
-                    st[kh][e] = p;
-                    psum += p;
+                    const int key = key0 + 32 * kh + 16 * (e / 8) + 8 * hb + (e % 8);
+                    st[kh][e] = key <= qpos ? st[kh][e] : -FLT_MAX;
                 }
-            psum += __shfl_xor(psum, 32);
-            l_run = l_run * alpha + psum;
-            // the running max settles after the first tiles: skip the rescale of O^T when no lane needs it
-            if (__builtin_amdgcn_ballot_w64(m_new != m_run) != 0) {
+        }
+    };
+    // first product of tile kt into st, optionally with the softmax of the previous tile (in prev) between
+    // its MFMAs; the first V fragments of the tile whose second product follows (in vt) ride on its last MFMAs
+    half8_t vf[LA];
+    auto qk = [&](float16_t (&st)[2], int kt, auto with_softmax, float16_t (&prev)[2], const half_t *vt) {
+        const half_t *ks = Ks + (kt & 1) * KTILE;
 #pragma unroll
-                for (int t = 0; t < DT; ++t)
+        for (int e = 0; e < 16; ++e) st[0][e] = st[1][e] = 0.f;
+        half8_t kf[LA];
 #pragma unroll
-                    for (int e = 0; e < 16; ++e) o[t][e] *= alpha;
-            }
-            m_run = m_new;
-
-            // O^T += V^T . P^T, four 16-key steps
+        for (int j = 0; j < LA; ++j)
+            if (j < NQ) kf[j] = kfrag(ks, j);
 #pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                half8_t pb;
+        for (int i = 0; i < NQ; ++i) {
+            st[i % 2] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[i % LA], qf[i / 2], st[i % 2], 0, 0, 0);
+            if (i + LA < NQ) kf[i % LA] = kfrag(ks, i + LA);
+            else if (vt && i + LA - NQ < LA && i + LA - NQ < NP) vf[i + LA - NQ] = vfrag(vt, i + LA - NQ);
+            if (decltype(with_softmax)::value) sm_slice(prev, i);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    // second product: O^T += V^T . P^T with P = st (fp16), V tile in vt; vf[0..LA) already hold its first fragments
+    auto pv = [&](float16_t (&st)[2], const half_t *vt) {
+        half8_t pb;
+#pragma unroll
+        for (int i = 0; i < NP; ++i) {
+            if (i % DT == 0) {
+                const int u = i / DT;
 #pragma unroll
                 for (int j = 0; j < 8; ++j) pb[j] = (half_t)st[u / 2][8 * (u % 2) + j];
-#pragma unroll
-                for (int t = 0; t < DT; ++t) {
-                    half8_t vf = load8(vt + (32 * t + n) * VLD + 16 * u + 8 * hb);
-                    o[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, pb, o[t], 0, 0, 0);
-                }
             }
+            o[i % DT] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf[i % LA], pb, o[i % DT], 0, 0, 0);
+            if (i + LA < NP) vf[i % LA] = vfrag(vt, i + LA);
+            __builtin_amdgcn_sched_barrier(0);
         }
-        if (kt + 1 < n_tiles) sstore(buf ^ 1);
+    };
+    auto load_vf = [&](const half_t *vt) {
+#pragma unroll
+        for (int j = 0; j < LA; ++j)
+            if (j < NP) vf[j] = vfrag(vt, j);
+    };
+
+    // Schedule.  K runs two tiles ahead of the tile being finished, V one: step t finishes tile t (softmax,
+    // second product) while the first product of tile t + 1 is computed between the softmax instructions,
+    // so the matrix pipe works under the softmax.  The last two tiles of the workgroup are the only ones
+    // that can need the causal mask or lie beyond a wavefront's rows; they take the plain path below.
+    //   LDS: K tile t in Ks[t & 1], V tile t in Vt[t & 1]; step t stores K(t + 2) and V(t + 1) at its end.
+    gload_k(0);
+    gload_v(0);
+    sstore_k(0);
+    sstore_v(0);
+    if (n_tiles > 1) {
+        gload_k(AP_BKEY);
+        sstore_k(1);
+    }
+    // All loads issued so far (the query fragments among them) are complete from here on.  Without this
+    // wait the compiler, which cannot tell the first pass of a loop from the others, makes every pass
+    // wait for the query registers with counts that also drain the K/V prefetch issued at its top.
+    __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0)
+    __syncthreads();
+
+    const int n_main = n_tiles > 2 ? n_tiles - 2 : 0;
+    float16_t sa[2], sb[2];
+    auto stage_in = [&](int kt) { // global loads of the tiles that step kt stores
+        if (kt + 2 < n_tiles) gload_k((kt + 2) * AP_BKEY);
+        if (kt + 1 < n_tiles) gload_v((kt + 1) * AP_BKEY);
+    };
+    auto stage_out = [&](int kt) {
+        if (kt + 2 < n_tiles) sstore_k(kt & 1);
+        if (kt + 1 < n_tiles) sstore_v((kt + 1) & 1);
         __syncthreads();
+    };
+    // main step on tile kt < n_main: scores of tile kt are in cur, those of tile kt + 1 go to nxt
+    auto step = [&](int kt, float16_t (&cur)[2], float16_t (&nxt)[2]) {
+        stage_in(kt);
+        if (live) {
+            const half_t *vt = Vt + (kt & 1) * VTILE;
+            qk(nxt, kt + 1, std::true_type{}, cur, vt);
+            sm_finish();
+            pv(cur, vt);
+        }
+        stage_out(kt);
+    };
+    if (live) qk(sa, 0, std::false_type{}, sa, (const half_t *)nullptr);
+    int kt = 0;
+    for (; kt + 1 < n_main; kt += 2) {
+        step(kt, sa, sb);
+        step(kt + 1, sb, sa);
+    }
+    if (kt < n_main) {
+        step(kt, sa, sb);
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            sa[0][e] = sb[0][e];
+            sa[1][e] = sb[1][e];
+        }
+        ++kt;
+    }
+    // plain path: tile kt has its scores in sa; the tile after it (if any) is computed here
+    for (; kt < n_tiles; ++kt) {
+        const int key0 = kt * AP_BKEY;
+        stage_in(kt);
+        if (live && key0 <= my_last) {
+            const half_t *vt = Vt + (kt & 1) * VTILE;
+            load_vf(vt);
+            mask(sa, key0);
+#pragma unroll
+            for (int i = 0; i < NQ; ++i) sm_slice(sa, i);
+            sm_finish();
+            pv(sa, vt);
+        }
+        if (kt + 1 < n_tiles && live && key0 + AP_BKEY <= my_last) qk(sa, kt + 1, std::false_type{}, sa, (const half_t *)nullptr);
+        stage_out(kt);
     }
 
     // O^T lane l: query q0 + l%32, dims 32t + 8*(e/4) + 4*(l/32) + e%4
