@@ -166,7 +166,9 @@ def test_swiglu_skinny(gpu, T):
 
 @pytest.mark.parametrize("T,K,N", [(17, 256, 384), (33, 768, 256), (64, 256, 768), (100, 4096, 512),
                                    (128, 4096, 6144), (200, 512, 1040), (129, 64, 272), (300, 128, 1008),
-                                   (1000, 256, 4112), (1025, 64, 272), (1100, 192, 528), (2100, 4096, 400)])
+                                   (1000, 256, 4112), (1025, 64, 272), (1100, 192, 528), (2100, 4096, 400),
+                                   # enough 256 x 256 tiles for the four-wave kernel, ragged edges, 2..6 k-steps
+                                   (1100, 128, 10000), (1030, 64, 12304), (1300, 192, 9232)])
 def test_linear_gemm_ragged_shapes(gpu, T, K, N):
     x, w = _proj_inputs(T + K + N, T, K, N)
     res = H.bits(np.random.default_rng(1).standard_normal((T, N)))
@@ -192,7 +194,8 @@ def test_linear_gemm_reference_test_operand_pattern(gpu):
     assert np.array_equal(gpu.ops.linear(H.bits(x[:5]), H.bits(w)), H.bits(x[:5] @ w.T))
 
 
-@pytest.mark.parametrize("T,K,N", [(130, 64, 80), (300, 512, 1008), (1030, 128, 336), (1500, 4096, 208)])
+@pytest.mark.parametrize("T,K,N", [(130, 64, 80), (300, 512, 1008), (1030, 128, 336), (1500, 4096, 208),
+                                   (1030, 128, 5008), (1500, 64, 4112)])
 def test_swiglu_gemm_ragged_shapes(gpu, T, K, N):
     rng = np.random.default_rng(T + N)
     x = H.bits(rng.standard_normal((T, K)))
