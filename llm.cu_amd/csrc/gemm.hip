@@ -909,6 +909,9 @@ int llm_linear(const uint16_t *x, int ldx, const uint16_t *w, const uint16_t *re
     if (T <= 128) {
         // weight-streaming regime: 128 x 128 tiles, k split so that every CU has work
         const long tiles = (long)((N + 127) / 128);
+        if (T <= 64) // 64-row tiles: half the x traffic of the 128-row tile
+            return gemm_dma_launch<1, 2, 1, 4, false, 2, 1>(xp, ldx, wp, nullptr, rp, ldr, op, ldo, T, N, K,
+                                                            pick_splits(tiles, T, N, K), s);
         return gemm_dma_launch<1, 2, 1, 4, false, 2>(xp, ldx, wp, nullptr, rp, ldr, op, ldo, T, N, K,
                                                      pick_splits(tiles, T, N, K), s);
     }
@@ -951,6 +954,9 @@ int llm_linear_swiglu(const uint16_t *x, int ldx, const uint16_t *wgate, const u
         return gemm_launch<128, 64, 2, 2, 2>(xp, ldx, gp, up, nullptr, 0, op, ldo, T, N, K, s);
     }
     // (splitting k here costs more in fp32 partial traffic than the extra workgroups return)
+    if (T <= 64)
+        return gemm_dma_launch<2, 2, 1, 4, false, 2, 1>(xp, ldx, gp, up, nullptr, 0, op, ldo, T, N, K,
+                                                        pick_splits(2 * (long)((N + 63) / 64), T, N, K, 2), s);
     if (T <= 128)
         return gemm_dma_launch<2, 2, 1, 4, false, 2>(xp, ldx, gp, up, nullptr, 0, op, ldo, T, N, K,
                                                      pick_splits(2 * (long)((N + 63) / 64), T, N, K, 2), s);
