@@ -312,7 +312,11 @@ def test_attn_decode_small_heads_and_gqa_map(gpu):
 
 
 @pytest.mark.parametrize("T,pos0,Hq,Hkv,hd", [(1, 0, 8, 2, 32), (16, 0, 8, 2, 32), (33, 7, 8, 2, 32),
-                                              (64, 0, 32, 8, 128), (100, 60, 32, 8, 128), (512, 0, 32, 8, 128)])
+                                              (64, 0, 32, 8, 128), (100, 60, 32, 8, 128), (512, 0, 32, 8, 128),
+                                              # several pipelined tiles before the masked ones, rows not a multiple of the
+                                              # block, prompt continued at an unaligned position; other group sizes and head dims
+                                              (300, 37, 32, 8, 128), (257, 129, 8, 2, 64), (200, 300, 8, 1, 128),
+                                              (130, 5, 4, 4, 128), (321, 64, 16, 4, 32)])
 def test_attn_prefill(gpu, T, pos0, Hq, Hkv, hd):
     P = pos0 + T
     q, k, v = _attn_inputs(T + pos0, P, Hq, Hkv, hd)
