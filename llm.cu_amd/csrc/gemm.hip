@@ -538,6 +538,18 @@ template <int N> __device__ __forceinline__ void dma_wait_barrier() {
     // vmcnt(N): all but the newest N of this wave's loads have landed; then the workgroup barrier.
     asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(N) : "memory");
 }
+// the same with a run-time number of tiles (of LPT loads each, at most MAXT) allowed to stay in flight
+template <int LPT, int MAXT> __device__ __forceinline__ void dma_wait_tiles(int tiles) {
+    static_assert(MAXT * LPT <= 63, "vmcnt counts at most 63 outstanding loads");
+    if (MAXT >= 7 && tiles >= 7) dma_wait_barrier<(MAXT >= 7 ? 7 : 0) * LPT>();
+    else if (MAXT >= 6 && tiles >= 6) dma_wait_barrier<(MAXT >= 6 ? 6 : 0) * LPT>();
+    else if (MAXT >= 5 && tiles >= 5) dma_wait_barrier<(MAXT >= 5 ? 5 : 0) * LPT>();
+    else if (MAXT >= 4 && tiles >= 4) dma_wait_barrier<(MAXT >= 4 ? 4 : 0) * LPT>();
+    else if (MAXT >= 3 && tiles >= 3) dma_wait_barrier<(MAXT >= 3 ? 3 : 0) * LPT>();
+    else if (MAXT >= 2 && tiles >= 2) dma_wait_barrier<(MAXT >= 2 ? 2 : 0) * LPT>();
+    else if (MAXT >= 1 && tiles >= 1) dma_wait_barrier<(MAXT >= 1 ? 1 : 0) * LPT>();
+    else dma_wait_barrier<0>();
+}
 
 // (WGM*FM*32) x (WGN*128) macro-tile, WGM*WGN wavefronts each owning (FM*32) x 128 of it (NB = 2: 64 columns of
 // gate and the same 64 of up), BK = 32, STAGES LDS buffers filled by direct global->LDS loads.
@@ -721,9 +733,7 @@ __global__ __launch_bounds__(WGM * WGN * 64, OCC) void gemm_dma_kernel(const hal
             // tile kt landed?  loads issued after it: tiles kt+1 .. min(kt+AHEAD-1, nk-1)
             const int last = kt + AHEAD - 1 < nk - 1 ? kt + AHEAD - 1 : nk - 1;
             const int beyond = last - kt;
-            if (AHEAD >= 3 && beyond >= 2) dma_wait_barrier<2 * LPT>();
-            else if (beyond >= 1) dma_wait_barrier<LPT>();
-            else dma_wait_barrier<0>();
+            dma_wait_tiles<LPT, AHEAD - 1>(beyond);
             if (kt + AHEAD < nk) issue(kt + AHEAD);
             lfrag(0, kt, 0);
             lfrag(1, kt, 1);
@@ -912,8 +922,9 @@ int llm_linear(const uint16_t *x, int ldx, const uint16_t *w, const uint16_t *re
         if (T <= 64) // 64-row tiles: half the x traffic of the 128-row tile
             return gemm_dma_launch<1, 2, 1, 4, false, 2, 1>(xp, ldx, wp, nullptr, rp, ldr, op, ldo, T, N, K,
                                                             pick_splits(tiles, T, N, K), s);
-        return gemm_dma_launch<1, 2, 1, 4, false, 2>(xp, ldx, wp, nullptr, rp, ldr, op, ldo, T, N, K,
-                                                     pick_splits(tiles, T, N, K), s);
+        // four waves of 32 rows rather than two of 64: with so few workgroups the MFMA work needs the SIMDs
+        return gemm_dma_launch<1, 4, 1, 4, false, 2, 1>(xp, ldx, wp, nullptr, rp, ldr, op, ldo, T, N, K,
+                                                        pick_splits(tiles, T, N, K), s);
     }
     // Measured at the 8B shapes: once the 256 x 256 tiles cover about three quarters of the CUs the
     // 4-wave tile below with its pinned, interleaved pipeline wins; with fewer tiles the 256 x 128 tile,
@@ -958,8 +969,8 @@ int llm_linear_swiglu(const uint16_t *x, int ldx, const uint16_t *wgate, const u
         return gemm_dma_launch<2, 2, 1, 4, false, 2, 1>(xp, ldx, gp, up, nullptr, 0, op, ldo, T, N, K,
                                                         pick_splits(2 * (long)((N + 63) / 64), T, N, K, 2), s);
     if (T <= 128)
-        return gemm_dma_launch<2, 2, 1, 4, false, 2>(xp, ldx, gp, up, nullptr, 0, op, ldo, T, N, K,
-                                                     pick_splits(2 * (long)((N + 63) / 64), T, N, K, 2), s);
+        return gemm_dma_launch<2, 4, 1, 4, false, 2, 1>(xp, ldx, gp, up, nullptr, 0, op, ldo, T, N, K,
+                                                        pick_splits(2 * (long)((N + 63) / 64), T, N, K, 2), s);
     if ((long)((T + 255) / 256) * ((N + 127) / 128) < 192)
         return gemm_dma_launch<2, 4, 1, 3, false, 2>(xp, ldx, gp, up, nullptr, 0, op, ldo, T, N, K, 1, s);
     return gemm_dma_launch<2, 2, 2, 4, true, 1, 4>(xp, ldx, gp, up, nullptr, 0, op, ldo, T, N, K, 1, s);
