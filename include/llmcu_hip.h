@@ -209,6 +209,10 @@ int llm_norm_lmhead_argmax(const uint16_t *x_dev, const uint16_t *gain_dev, doub
 /* argmax alone over fp16 values (same tie/NaN rule); workspace as for the LM head of n rows. */
 int llm_argmax_f16(const uint16_t *logits_dev, int n, int32_t *token_dev, void *workspace_dev,
                    llm_stream_t stream);
+/* The same for every row of a [rows, ld] matrix in two launches: tokens_dev[r] = argmax of row r.
+ * workspace_dev: rows * min(1024, ceil(n / 256)) * 8 bytes. */
+int llm_argmax_f16_rows(const uint16_t *logits_dev, int ld, int rows, int n, int32_t *tokens_dev,
+                        void *workspace_dev, llm_stream_t stream);
 
 #ifdef __cplusplus
 }

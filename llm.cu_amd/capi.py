@@ -125,6 +125,7 @@ HIP_ABI = {
     "llm_lmhead_workspace_bytes": (_sz, [_i]),
     "llm_lmhead_argmax": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp, _vp]),
     "llm_argmax_f16": (_i, [_vp, _i, _vp, _vp, _vp]),
+    "llm_argmax_f16_rows": (_i, [_vp, _i, _i, _i, _vp, _vp, _vp]),
 }
 _LP, _CP = C.POINTER(Llama3), C.POINTER(CudaCache)
 HOST_ABI = {

@@ -172,10 +172,13 @@ __global__ __launch_bounds__(GEMV_THREADS) void gemv_kernel(const GemvArgs a) {
 }
 
 // candidates over plain fp16 values (argmax alone)
+// (blockIdx.y: row of a [rows, ld] matrix; its candidates follow those of the rows before it)
 __global__ __launch_bounds__(256) void argmax_candidates_kernel(const half_t *__restrict__ v, int n,
-                                                                unsigned long long *__restrict__ cand) {
+                                                                unsigned long long *__restrict__ cand, int ld) {
     __shared__ unsigned long long best[256];
     unsigned long long mine = 0ull;
+    v += (size_t)blockIdx.y * ld;
+    cand += (size_t)blockIdx.y * gridDim.x;
     for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x) {
         unsigned long long c = pack_candidate(v[i], i);
         mine = c > mine ? c : mine;
@@ -196,6 +199,8 @@ __global__ __launch_bounds__(1024) void argmax_final_kernel(const unsigned long 
                                                             int32_t *__restrict__ pos) {
     __shared__ unsigned long long best[1024];
     unsigned long long mine = 0ull;
+    cand += (size_t)blockIdx.x * n; // one block per row
+    token += blockIdx.x;
     for (int i = threadIdx.x; i < n; i += 1024) mine = cand[i] > mine ? cand[i] : mine;
     best[threadIdx.x] = mine;
     __syncthreads();
@@ -282,19 +287,24 @@ int llm_lmhead_argmax(const uint16_t *x, const uint16_t *w, uint16_t *logits, in
     return llm_norm_lmhead_argmax(x, nullptr, 0.0, w, logits, token, tokens, pos, vocab, K, workspace, stream);
 }
 
-int llm_argmax_f16(const uint16_t *logits, int n, int32_t *token, void *workspace, llm_stream_t stream) {
-    LLM_REQUIRE(logits && token && workspace, "llm_argmax_f16: null pointer");
-    LLM_REQUIRE(n > 0, "llm_argmax_f16: n=%d", n);
+int llm_argmax_f16_rows(const uint16_t *logits, int ld, int rows, int n, int32_t *tokens, void *workspace,
+                        llm_stream_t stream) {
+    LLM_REQUIRE(logits && tokens && workspace, "llm_argmax_f16: null pointer");
+    LLM_REQUIRE(n > 0 && rows > 0 && rows <= 65535 && ld >= n, "llm_argmax_f16: rows=%d n=%d ld=%d", rows, n, ld);
     hipStream_t s = (hipStream_t)stream;
     int blocks = (n + 255) / 256;
     if (blocks > 1024) blocks = 1024;
-    argmax_candidates_kernel<<<dim3(blocks), dim3(256), 0, s>>>((const half_t *)logits, n,
-                                                                (unsigned long long *)workspace);
+    argmax_candidates_kernel<<<dim3(blocks, rows), dim3(256), 0, s>>>((const half_t *)logits, n,
+                                                                      (unsigned long long *)workspace, ld);
     LLM_LAUNCH_CHECK("argmax_candidates_kernel");
-    argmax_final_kernel<<<dim3(1), dim3(1024), 0, s>>>((const unsigned long long *)workspace, blocks, token, nullptr,
-                                                       nullptr);
+    argmax_final_kernel<<<dim3(rows), dim3(1024), 0, s>>>((const unsigned long long *)workspace, blocks, tokens, nullptr,
+                                                          nullptr);
     LLM_LAUNCH_CHECK("argmax_final_kernel");
     return LLM_OK;
+}
+
+int llm_argmax_f16(const uint16_t *logits, int n, int32_t *token, void *workspace, llm_stream_t stream) {
+    return llm_argmax_f16_rows(logits, n, 1, n, token, workspace, stream);
 }
 
 } // extern "C"

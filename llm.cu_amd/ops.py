@@ -156,6 +156,16 @@ def argmax_f16(logits):
     return int(d_t.download()[0])
 
 
+def argmax_f16_rows(logits):
+    """argmax of every row of a 2-D fp16 array in one call."""
+    logits = _u16(logits)
+    rows, n = logits.shape
+    d_l, d_t = DevBuf.from_host(logits), DevBuf((rows,), np.int32)
+    d_ws = DevBuf((rows * min(1024, (n + 255) // 256) * 8,), np.uint8)
+    check(lib().llm_argmax_f16_rows(d_l.ptr, n, rows, n, d_t.ptr, d_ws.ptr, None))
+    return d_t.download()
+
+
 class Timer:
     """HIP-event timing of repeated launches on one stream."""
 

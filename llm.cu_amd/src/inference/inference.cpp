@@ -58,7 +58,7 @@ struct Engine {
     int batch_cap = 0;
     llm_half *b_logits = nullptr; // [batch][vocab]
     int32_t *b_ids = nullptr;     // [batch] input ids, then the argmax results
-    void *b_ws_attn = nullptr;
+    void *b_ws_attn = nullptr, *b_ws_argmax = nullptr;
     llm_event_t ev[4] = {nullptr, nullptr, nullptr, nullptr};
 };
 
@@ -346,7 +346,7 @@ extern "C" void free_cache(CudaCache *C) {
         drop_graph(e);
         void *bufs[] = {e->x, e->xn, e->qkv, e->attn, e->ffn, e->logits, e->kc, e->vc, e->rope_table,
                         e->d_tokens, e->d_pos, e->d_token, e->ws_attn, e->ws_lm, e->trace_dev, e->inject_dev,
-                        e->b_logits, e->b_ids, e->b_ws_attn};
+                        e->b_logits, e->b_ids, e->b_ws_attn, e->b_ws_argmax};
         for (void *b : bufs) llm_free(b);
         for (auto ev : e->ev) llm_event_destroy(ev);
         llm_stream_destroy(e->stream);
@@ -484,11 +484,13 @@ extern "C" void llama3_decode_batch(Llama3 *m, CudaCache *const *caches, const i
         if (e0->b_logits) llm_free(e0->b_logits);
         if (e0->b_ids) llm_free(e0->b_ids);
         if (e0->b_ws_attn) llm_free(e0->b_ws_attn);
+        if (e0->b_ws_argmax) llm_free(e0->b_ws_argmax);
         e0->b_logits = dmalloc<llm_half>((size_t)16 * c.vocab, "llm_malloc(batch logits)");
         e0->b_ids = dmalloc<int32_t>(16, "llm_malloc(batch ids)");
         const size_t wsb = llm_attn_decode_workspace_bytes(Hq, hd);
         e0->b_ws_attn = dmalloc<char>(wsb * 16, "llm_malloc(batch attention workspace)");
         llama3_check(llm_fill_zero(e0->b_ws_attn, wsb * 16, s), "zero workspace");
+        e0->b_ws_argmax = dmalloc<char>((size_t)16 * 1024 * 8, "llm_malloc(batch argmax candidates)");
         e0->batch_cap = 16;
     }
     llama3_check(llm_memcpy_h2d(e0->b_ids, tokens, sizeof(int32_t) * (size_t)batch, s), "H2D ids");
@@ -520,9 +522,8 @@ extern "C" void llama3_decode_batch(Llama3 *m, CudaCache *const *caches, const i
     llama3_check(llm_rmsnorm(e0->x, m->norm->d_fp16_tensor, e0->xn, batch, d, c.rms_eps, s), "llm_rmsnorm");
     llama3_check(llm_linear(e0->xn, d, m->lm_head->d_fp16_tensor, nullptr, 0, e0->b_logits, c.vocab, batch, c.vocab, d, s),
                  "llm_linear(lm_head)");
-    for (int b = 0; b < batch; ++b)
-        llama3_check(llm_argmax_f16(e0->b_logits + (size_t)b * c.vocab, c.vocab, e0->b_ids + b, e0->ws_lm, s),
-                     "llm_argmax_f16");
+    llama3_check(llm_argmax_f16_rows(e0->b_logits, c.vocab, batch, c.vocab, e0->b_ids, e0->b_ws_argmax, s),
+                 "llm_argmax_f16_rows");
     int32_t out[16];
     llama3_check(llm_memcpy_d2h(out, e0->b_ids, sizeof(int32_t) * (size_t)batch, s), "D2H tokens");
     llama3_check(llm_stream_sync(s), "stream sync");

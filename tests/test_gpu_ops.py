@@ -276,6 +276,14 @@ def test_argmax_ties_zero_signs_nan(gpu):
         assert gpu.ops.argmax_f16(c) == orc.argmax_f16(c)
 
 
+@pytest.mark.parametrize("rows,n", [(1, 5), (4, 4096), (16, 128256), (3, 300001)])
+def test_argmax_rows_matches_row_by_row(gpu, rows, n):
+    rng = np.random.default_rng(rows * 1000 + n)
+    m = H.bits(np.round(rng.standard_normal((rows, n)) * 8) / 8)  # many ties: the lowest index must win in every row
+    got = gpu.ops.argmax_f16_rows(m)
+    assert list(got) == [orc.argmax_f16(m[r]) for r in range(rows)]
+
+
 # ---- attention ----------------------------------------------------------------------------------------------------
 def _attn_inputs(seed, P, Hq, Hkv, hd):
     rng = np.random.default_rng(seed)
