@@ -25,8 +25,7 @@ int gemv_swiglu_launch(const half_t *x, const half_t *gain, double eps, const ha
 
 __device__ __forceinline__ float silu_g(float g) { return g / (1.0f + expf(-g)); }
 
-// address-space casts for __builtin_amdgcn_global_load_lds (global memory straight into LDS)
-#define DMA_GP(p) ((const __attribute__((address_space(1))) void *)(p))
+// address-space cast for the LDS side of the loads that go from global memory straight into LDS
 #define DMA_LP(p) ((__attribute__((address_space(3))) void *)(p))
 
 // ---------------------------------------------------------------------------
@@ -526,8 +525,8 @@ static int gemm_launch(const half_t *x, int ldx, const half_t *w, const half_t *
 // ---------------------------------------------------------------------------
 // large-T MFMA GEMM: tiles go from global memory straight into LDS
 // ---------------------------------------------------------------------------
-// No register staging: every wavefront issues global_load_lds (16 B per lane, 1 KB per instruction,
-// landing contiguously in LDS), STAGES buffers deep, and waits with an explicit vmcnt so that loads
+// No register staging: every wavefront issues buffer loads with LDS destination (16 B per lane, 1 KB per
+// instruction, landing contiguously in LDS), STAGES buffers deep, and waits with an explicit vmcnt so that loads
 // stay in flight across workgroup barriers.  Because a wave instruction fills 16 consecutive 64-byte
 // rows, the row padding of the kernel above is not available; instead lane l fetches global 16-byte
 // chunk (l%4) ^ ((row>>2)&3) of its row, so that the 16 lanes an LDS read serves per cycle (16 rows,
