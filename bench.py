@@ -122,14 +122,18 @@ def main():
         p8k = eng_mod.seeded_tokens(a.seed + 1, T, cfg.vocab)
         engine.reset()
         engine.generate(p8k, 1)  # warm-up (first use of the large-tile kernels)
-        engine.reset()
-        _, st8 = engine.generate(p8k, 1)
-        sec = st8.prefill_ms * 1e-3
-        prefill = {"tokens": T, "ms": st8.prefill_ms, "tok_per_s": T / sec,
+        passes = []
+        for _ in range(3):  # median of three timed passes
+            engine.reset()
+            _, st8 = engine.generate(p8k, 1)
+            passes.append(st8.prefill_ms)
+        ms8 = sorted(passes)[1]
+        sec = ms8 * 1e-3
+        prefill = {"tokens": T, "ms": ms8, "passes_ms": passes, "tok_per_s": T / sec,
                    "flops": prefill_flops(T), "mfma_frac": prefill_flops(T) / sec / MFMA_F16_PEAK,
                    "peak_tflops": MFMA_F16_PEAK / 1e12}
         log("prefill 8192: %.1f ms -> %.0f tok/s (%.1f%% of fp16 MFMA peak)"
-            % (st8.prefill_ms, T / sec, 100 * prefill["mfma_frac"]))
+            % (ms8, T / sec, 100 * prefill["mfma_frac"]))
         # long-context decode (KV streaming next to weight streaming), 64 steps at ctx ~8.2K
         engine.reset()
         _, stl = engine.generate(p8k, 65)
