@@ -144,6 +144,7 @@ __global__ __launch_bounds__(G *AP_QT * 64) void attn_prefill_kernel(const half_
     // sm_finish adds the row sum into l_run and rescales O^T if some lane's max moved.  The softmax runs in
     // base 2: with c2 = log2(e)/sqrt(hd), p is one fma and one v_exp_f32 per score.
     float sm_mx = -FLT_MAX, sm_new = 0.f, sm_alpha = 1.f, sm_sum = 0.f;
+    half2_t pk[16]; // the 32 probabilities of the tile whose softmax ran last, as fp16 pairs
     auto sm_slice = [&](float16_t (&st)[2], int i) {
         constexpr int PM = 128 / NQ, PE = 64 / NQ; // scores per max slice / per exp slice
         if (i < NQ / 4) {
@@ -162,12 +163,18 @@ __global__ __launch_bounds__(G *AP_QT * 64) void attn_prefill_kernel(const half_
             sm_sum = 0.f;
         }
         if (i >= NQ / 2) {
+            // probabilities are rounded to fp16 here (the second product takes them in fp16) and the row sum
+            // is taken over the rounded values, two per v_dot2_f32_f16: numerator and denominator of the
+            // output then use the same weights, and the sum costs half the instructions
+            static_assert(PE % 2 == 0, "pairs");
 #pragma unroll
-            for (int j = 0; j < PE; ++j) {
+            for (int j = 0; j < PE; j += 2) {
                 const int e = (i - NQ / 2) * PE + j;
-                const float p = __builtin_amdgcn_exp2f(fmaf(st[e / 16][e % 16], c2, -sm_new));
-                st[e / 16][e % 16] = p;
-                sm_sum += p;
+                const float p0 = __builtin_amdgcn_exp2f(fmaf(st[e / 16][e % 16], c2, -sm_new));
+                const float p1 = __builtin_amdgcn_exp2f(fmaf(st[(e + 1) / 16][(e + 1) % 16], c2, -sm_new));
+                const half2_t h = {(half_t)p0, (half_t)p1};
+                pk[e / 2] = h;
+                sm_sum = __builtin_amdgcn_fdot2(h, half2_t{(half_t)1.0f, (half_t)1.0f}, sm_sum, false);
             }
         }
     };
@@ -225,7 +232,7 @@ __global__ __launch_bounds__(G *AP_QT * 64) void attn_prefill_kernel(const half_
             if (i % DT == 0) {
                 const int u = i / DT;
 #pragma unroll
-                for (int j = 0; j < 8; ++j) pb[j] = (half_t)st[u / 2][8 * (u % 2) + j];
+                for (int j = 0; j < 8; ++j) pb[j] = pk[(u / 2) * 8 + 4 * (u % 2) + j / 2][j % 2];
             }
             o[i % DT] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf[i % LA], pb, o[i % DT], 0, 0, 0);
             if (i + LA < NP) vf[i % LA] = vfrag(vt, i + LA);
