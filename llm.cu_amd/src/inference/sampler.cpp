@@ -134,12 +134,16 @@ int sample_next_token(float *tensor, llm_half *half_tensor) {
     const int k = g_top_k;
     if (k <= 0 || k >= g_vocab || !(g_top_p > 0.0f) || g_top_p > 0.99f)
         return sample_next_token_reference(tensor, half_tensor);
+    // the exponentials are independent (any thread gives the same bits); their sum is taken afterwards in
+    // index order, as the reference's single loop does
+    const int vocab = g_vocab;
+    const float temperature = g_temperature;
+#pragma omp parallel for schedule(static)
+    for (int i = 0; i < vocab; ++i) tensor[i] = expf(half_to_float(half_tensor[i]) / temperature);
     float cumsum = 0.0f;
-    for (int i = 0; i < g_vocab; ++i) {
-        tensor[i] = expf(half_to_float(half_tensor[i]) / g_temperature);
-        cumsum += tensor[i];
-    }
-    for (int i = 0; i < g_vocab; ++i) tensor[i] /= cumsum;
+    for (int i = 0; i < vocab; ++i) cumsum += tensor[i];
+#pragma omp parallel for schedule(static)
+    for (int i = 0; i < vocab; ++i) tensor[i] /= cumsum;
     // NaN probabilities (exp overflow) defeat every comparison: let the reference path decide
     if (!(cumsum < INFINITY) || !(cumsum > 0.0f)) return sample_next_token_reference(tensor, half_tensor);
     // k largest by (probability desc, index asc): threshold pass, then a sort of the few survivors
