@@ -222,3 +222,54 @@ def attention_f64(q, k, v, pos0, n_heads, n_kv_heads, head_dim):
 
 def silu(x):
     return x / (1.0 + np.exp(-x))
+
+
+def model_forward_f64(cfg, w, tokens, mutate=None):
+    """Independent float64 forward of the whole model, composed from the closed forms above and
+    plain `@`, wired as the reference's driver is (src/inference/inference.cu:149-193): embedding;
+    per layer  x += Wo.attn(rope(Wq.n), rope(Wk.n), Wv.n) with n = norm(x, input_ln),  then
+    x += Wdown.(silu(Wgate.m) * (Wup.m)) with m = norm(x, post_ln);  final norm; LM head on the last
+    row only (inference.cu:1014).  No intermediate rounding.  Returns (hidden [L,T,d], logits [V]).
+    `mutate` names one deliberate wiring mistake, used to show that the comparison would catch it."""
+    d, Hq, Hkv, hd = cfg["d_model"], cfg["n_heads"], cfg["n_kv_heads"], cfg["head_dim"]
+    eps, theta = cfg.get("rms_eps", 1e-5), cfg.get("rope_theta", 500000.0)
+    W = lambda a: f16(a)
+    norm = lambda x, g: x * W(g) / np.sqrt(eps + np.mean(x * x, axis=-1, keepdims=True))
+    T = len(tokens)
+
+    def rope(x, n_heads):
+        x = x.reshape(T, n_heads, hd // 2, 2)
+        ang = np.arange(T, dtype=np.float64)[:, None] * theta ** (-2.0 * np.arange(hd // 2) / hd)[None, :]
+        c, s = np.cos(ang)[:, None, :], np.sin(ang)[:, None, :]
+        return np.stack([c * x[..., 0] - s * x[..., 1], s * x[..., 0] + c * x[..., 1]], -1).reshape(T, n_heads * hd)
+
+    def attention(q, k, v):
+        out = np.zeros((T, Hq * hd))
+        for h in range(Hq):
+            kv = h // (Hq // Hkv)
+            s = q[:, h * hd:(h + 1) * hd] @ k[:, kv * hd:(kv + 1) * hd].T / np.sqrt(hd)
+            s = np.where(np.tril(np.ones((T, T), bool)), s, -np.inf)
+            p = np.exp(s - s.max(axis=1, keepdims=True))
+            out[:, h * hd:(h + 1) * hd] = (p / p.sum(axis=1, keepdims=True)) @ v[:, kv * hd:(kv + 1) * hd]
+        return out
+
+    x = W(w["embed"])[np.asarray(tokens)]
+    hidden = []
+    for l in range(cfg["n_layers"]):
+        g_in, g_post = w["input_ln"][l], w["post_ln"][l]
+        if mutate == "swap_norm_gains":
+            g_in, g_post = g_post, g_in
+        n = norm(x, g_in)
+        q, k, v = n @ W(w["wq"][l]).T, n @ W(w["wk"][l]).T, n @ W(w["wv"][l]).T
+        if mutate != "no_rope":
+            q, k = rope(q, Hq), rope(k, Hkv)
+        a = attention(q, k, v) @ W(w["wo"][l]).T
+        x = (n if mutate == "residual_after_norm" else x) + a
+        m = norm(x, g_post)
+        gate, up = m @ W(w["wgate"][l]).T, m @ W(w["wup"][l]).T
+        if mutate == "swap_gate_up":
+            gate, up = up, gate
+        x = x + (silu(gate) * up) @ W(w["wdown"][l]).T
+        hidden.append(x.copy())
+    last = x[-1] if mutate == "no_final_norm" else norm(x[-1:], w["norm"])[0]
+    return np.stack(hidden), last @ W(w["lm_head"]).T

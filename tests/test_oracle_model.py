@@ -6,6 +6,7 @@ import json
 import os
 
 import numpy as np
+import pytest
 
 from oracle import pyoracle as orc
 from tests import helpers as H
@@ -87,3 +88,76 @@ def test_golden_fixture(pkg):
     assert toks == g["tokens"]
     assert [int(hid[l].astype(np.uint64).sum()) for l in range(cfg.n_layers)] == g["hidden_bit_sums"]
     assert int(logits.astype(np.uint64).sum()) == g["logits_bit_sum"]
+
+
+# ---- the wiring of the whole model, against an independent float64 forward ------------------
+def _distinct_gain_weights(w, cfg, seed):
+    """The seeded tiny model has unit norm gains; give every norm its own random gains so that a
+    norm applied with the wrong gains (or not at all) changes the result."""
+    rng = np.random.default_rng(seed)
+    w = dict(w)
+    gain = lambda: H.bits(rng.uniform(0.5, 1.5, cfg.d_model))
+    w["input_ln"] = [gain() for _ in range(cfg.n_layers)]
+    w["post_ln"] = [gain() for _ in range(cfg.n_layers)]
+    w["norm"] = gain()
+    return w
+
+
+def _rel_err(a, b):
+    return float(np.max(np.abs(a - b) / (1.0 + np.abs(b))))
+
+
+def test_model_wiring_vs_independent_float64_forward(pkg):
+    """orc_model_forward (ORC_FP32: the same graph as ORC_REF16 without intermediate rounding) against
+    tests/helpers.model_forward_f64, which is written from the reference driver
+    (src/inference/inference.cu:149-193, LM head on the last row :1014) out of numpy closed forms and
+    shares no code with oracle.c.  Per-layer hidden states and logits within 1e-3, same argmax; then
+    ORC_REF16 within the model tolerance of the same float64 result."""
+    cfg, cd, w, prompt = _setup(pkg)
+    w = _distinct_gain_weights(w, cfg, 7)
+    hid64, lg64 = H.model_forward_f64(cd, w, [int(t) for t in prompt])
+    m = orc.Model(cd, w, orc.ORC_FP32)
+    tok, hid, lg = m.forward(prompt, want_hidden=True)
+    for l in range(cfg.n_layers):
+        assert _rel_err(H.f16(hid[l]), hid64[l]) < 1e-3, l   # fp16 export of an fp32 state: 2^-11 relative
+    assert _rel_err(H.f16(lg), lg64) < 1e-3
+    assert tok == int(np.argmax(lg64))
+    m16 = orc.Model(cd, w, orc.ORC_REF16)
+    tok16, hid16, lg16 = m16.forward(prompt, want_hidden=True)
+    assert max(_rel_err(H.f16(hid16[l]), hid64[l]) for l in range(cfg.n_layers)) < H.TOL
+    assert _rel_err(H.f16(lg16), lg64) < H.TOL
+    assert tok16 == int(np.argmax(lg64))
+    # decode steps through the KV cache against the float64 forward of the grown sequence
+    seq = [int(t) for t in prompt] + [tok]
+    for _ in range(3):
+        t, h1, lg = m.forward([seq[-1]], want_hidden=True)
+        hid64, lg64 = H.model_forward_f64(cd, w, seq)
+        assert _rel_err(H.f16(h1[:, 0, :]), hid64[:, -1, :]) < 1e-3
+        assert _rel_err(H.f16(lg), lg64) < 1e-3 and t == int(np.argmax(lg64))
+        seq.append(t)
+
+
+@pytest.mark.parametrize("mistake", ["swap_norm_gains", "residual_after_norm", "no_final_norm",
+                                     "swap_gate_up", "no_rope"])
+def test_wiring_check_is_sensitive_to_plausible_mistakes(pkg, mistake):
+    """The comparison above would fail for each plausible wiring mistake: the float64 forward with the
+    mistake built in is far outside 1e-3 of the oracle."""
+    cfg, cd, w, prompt = _setup(pkg)
+    w = _distinct_gain_weights(w, cfg, 7)
+    m = orc.Model(cd, w, orc.ORC_FP32)
+    _, hid, lg = m.forward(prompt, want_hidden=True)
+    hid_bad, lg_bad = H.model_forward_f64(cd, w, [int(t) for t in prompt], mutate=mistake)
+    worst = max(_rel_err(H.f16(lg), lg_bad), max(_rel_err(H.f16(hid[l]), hid_bad[l]) for l in range(cfg.n_layers)))
+    assert worst > 1e-2, (mistake, worst)
+
+
+def test_single_layer_model_wiring(pkg):
+    """One layer, distinct gains: nothing can hide behind a second layer."""
+    cfg, cd, w, prompt = _setup(pkg)
+    w = _distinct_gain_weights(w, cfg, 11)
+    cd1 = dict(cd, n_layers=1)
+    w1 = {k: (v[:1] if isinstance(v, list) else v) for k, v in w.items()}
+    hid64, lg64 = H.model_forward_f64(cd1, w1, [int(t) for t in prompt])
+    tok, hid, lg = orc.Model(cd1, w1, orc.ORC_FP32).forward(prompt, want_hidden=True)
+    assert _rel_err(H.f16(hid[0]), hid64[0]) < 1e-3 and _rel_err(H.f16(lg), lg64) < 1e-3
+    assert tok == int(np.argmax(lg64))

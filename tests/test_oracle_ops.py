@@ -106,6 +106,31 @@ def test_rmsnorm_rejects_non_power_of_two():
         orc.rmsnorm(np.zeros((1, 24), np.uint16), np.zeros(24, np.uint16))
 
 
+# ---- residual add ------------------------------------------------------------------------------
+def test_add_is_fp32_sum_rounded_once_to_fp16():
+    """orc_add (reference add_norm, src/inference/inference.cu:377-390): fp16(float(x) + float(res)).
+    Against numpy float32 on random values and on every pair from a set of edge patterns (signed
+    zeros, subnormals, the largest finite value, infinities); the fp32 sum of two fp16 values is
+    exact, so the result is the correctly rounded fp16 sum and float64 gives the same bits."""
+    rng = np.random.default_rng(12)
+    x = H.bits(rng.standard_normal(4099) * rng.choice([1e-4, 1.0, 300.0], 4099))
+    r = H.bits(rng.standard_normal(4099) * rng.choice([1e-4, 1.0, 300.0], 4099))
+    edge = np.array([0x0000, 0x8000, 0x0001, 0x8001, 0x03ff, 0x0400, 0x3c00, 0xbc00, 0x3c01, 0x7bff,
+                     0xfbff, 0x7c00, 0xfc00, 0x1400, 0x6800], np.uint16)
+    x = np.concatenate([x, np.repeat(edge, edge.size)])
+    r = np.concatenate([r, np.tile(edge, edge.size)])
+    got = orc.add(x, r)
+    with np.errstate(over="ignore", invalid="ignore"):
+        want32 = (x.view(np.float16).astype(np.float32) + r.view(np.float16).astype(np.float32)).astype(np.float16)
+        want64 = (x.view(np.float16).astype(np.float64) + r.view(np.float16).astype(np.float64)).astype(np.float16)
+    nan = np.isnan(want32)
+    assert np.array_equal(got[~nan], want32.view(np.uint16)[~nan])
+    assert np.array_equal(got[~nan], want64.view(np.uint16)[~nan])
+    assert np.all(np.isnan(got[nan].view(np.float16)))       # Inf + -Inf
+    assert orc.add(np.array([0x3c00], np.uint16), np.array([0x1000], np.uint16))[0] == 0x3c00  # 1 + half an ulp: tie to even
+    assert orc.add(np.array([0x3c01], np.uint16), np.array([0x1000], np.uint16))[0] == 0x3c02  # odd mantissa: the tie rounds up
+
+
 # ---- GEMM ----------------------------------------------------------------------------------
 def test_linear_reference_gemm_test_operands_closed_form():
     # tests/gemm.cu:63-105 of the reference: X[8x8], Transform[4x8], A[i][j] = i*cols + j,
