@@ -23,6 +23,22 @@ def mixed_err(a_bits, b_bits):
     return float(np.max(np.abs(a - b) / (1.0 + np.abs(b)))) if a.size else 0.0
 
 
+def same_pick_or_near_tie(lg_gpu, lg_orc, t_gpu, t_orc):
+    """Greedy ids on identical context: equal, or the oracle's own logits of the two ids are no
+    further apart than the engine's measured error at exactly those two logits (which the caller
+    bounds by the tolerance separately)."""
+    if int(t_gpu) == int(t_orc):
+        return True
+    g, o = f16(lg_gpu), f16(lg_orc)
+    return float(o[t_orc] - o[t_gpu]) <= float(abs(g[t_orc] - o[t_orc]) + abs(g[t_gpu] - o[t_gpu]))
+
+
+def rms_err(a_bits, b_bits):
+    """root mean square of a-b over the root mean square of b."""
+    a, b = f16(a_bits), f16(b_bits)
+    return float(np.sqrt(np.mean((a - b) ** 2) / max(np.mean(b * b), 1e-30)))
+
+
 def ulp_diff(a_bits, b_bits):
     """distance in fp16 ulps (monotone integer mapping of the bit patterns)."""
     def key(x):
@@ -121,7 +137,10 @@ def run_forced_parity(pkg, cfg, seed, n_prompt, n_decode):
       free_*    the engine runs on its own, errors compound;
       floor_*   ORC_REF16 against ORC_REF16_REV (the oracle with every projection summed over k in
                 the opposite order): what a legal fp32 reordering of the reference's own arithmetic
-                does to the same hidden states."""
+                does to the same hidden states;
+      exact_*   distance of each of the three (ORC_REF16, ORC_REF16_REV, the free-running engine) from
+                ORC_FP32, the same graph with no intermediate rounding: how close each rounding
+                schedule stays to exact arithmetic."""
     eng_mod = pkg.engine
     model = eng_mod.Model.seeded(cfg, seed)
     w = oracle_weights(model)
@@ -138,8 +157,19 @@ def run_forced_parity(pkg, cfg, seed, n_prompt, n_decode):
     out["floor_hidden_err"] = [mixed_err(hid_r[l], hid_o[l]) for l in range(L)]
     out["floor_logits_err"] = mixed_err(lg_r, lg_o)
     o_rev.close()
+    o_x = orc.Model(cfg_dict(cfg), w, orc.ORC_FP32)
+    _, hid_x, lg_x = o_x.forward(prompt, want_hidden=True)
+    o_x.close()
+    out["exact_err_ref16"] = [mixed_err(hid_o[l], hid_x[l]) for l in range(L)]
+    out["exact_err_rev"] = [mixed_err(hid_r[l], hid_x[l]) for l in range(L)]
+    out["exact_rms_ref16"] = [rms_err(hid_o[l], hid_x[l]) for l in range(L)]
+    out["exact_rms_rev"] = [rms_err(hid_r[l], hid_x[l]) for l in range(L)]
+    out["exact_logits_err_ref16"] = mixed_err(lg_o, lg_x)
     # free running
     tok_f, hid_f = engine.prefill(prompt, want_hidden=True)
+    out["exact_err_hip"] = [mixed_err(hid_f[l], hid_x[l]) for l in range(L)]
+    out["exact_rms_hip"] = [rms_err(hid_f[l], hid_x[l]) for l in range(L)]
+    out["exact_logits_err_hip"] = mixed_err(engine.logits(), lg_x)
     out["free_hidden_err"] = [mixed_err(hid_f[l], hid_o[l]) for l in range(L)]
     out["free_logits_err"] = mixed_err(engine.logits(), lg_o)
     out["free_first_token"] = (int(tok_f), int(tok_o))
@@ -150,9 +180,10 @@ def run_forced_parity(pkg, cfg, seed, n_prompt, n_decode):
     out["forced_hidden_err"] = [mixed_err(hid_g[l], hid_o[l]) for l in range(L)]
     out["forced_logits_err"] = [mixed_err(lg_g, lg_o)]
     # teacher forced greedy steps: both sides consume the oracle's tokens
-    toks_o, toks_g, gaps, dec_err = [int(tok_o)], [int(tok_g)], [], []
+    toks_o, toks_g, gaps, dec_err, pick_err, lg_steps = [int(tok_o)], [int(tok_g)], [], [], [], [lg_o]
     top = f16(lg_o)
     gaps.append(float(top.max() - top[tok_g]))
+    pick_err.append(float(abs(f16(lg_g)[tok_o] - top[tok_o]) + abs(f16(lg_g)[tok_g] - top[tok_g])))
     for _ in range(n_decode - 1):
         t_o, h_o, lg_o = o.forward([toks_o[-1]], want_hidden=True)
         t_g, h_g = engine.decode(toks_o[-1], want_hidden=True, inject=h_o)
@@ -161,10 +192,13 @@ def run_forced_parity(pkg, cfg, seed, n_prompt, n_decode):
         out["forced_logits_err"].append(mixed_err(lg_g, lg_o))
         top = f16(lg_o)
         gaps.append(float(top.max() - top[t_g]))  # 0 when both picked the same id
+        pick_err.append(float(abs(f16(lg_g)[t_o] - top[t_o]) + abs(f16(lg_g)[t_g] - top[t_g])))
+        lg_steps.append(lg_o)
         toks_o.append(int(t_o))
         toks_g.append(int(t_g))
     out["forced_decode_hidden_err"] = dec_err
     out["tokens_oracle"], out["tokens_gpu_forced"], out["forced_gap_at_pick"] = toks_o, toks_g, gaps
+    out["forced_pick_err"] = pick_err  # |engine - oracle| logit error summed over the two ids picked
     # free-running greedy tokens (device-resident loop) for the record
     engine.close()
     engine = eng_mod.Engine(model, cfg, use_graph=True)
@@ -176,6 +210,14 @@ def run_forced_parity(pkg, cfg, seed, n_prompt, n_decode):
             break
         same += 1
     out["free_identical_prefix"] = same
+    # at the first step where the free-running ids part, both sides still had identical context:
+    # how far apart the oracle itself holds the two ids there
+    if same < len(toks_o):
+        top = f16(lg_steps[same])
+        out["free_divergence_gap"] = float(top[toks_o[same]] - top[out["tokens_gpu_free"][same]])
+        out["free_divergence_logit_scale"] = float(np.abs(top).max())
+    else:
+        out["free_divergence_gap"] = 0.0
     o.close()
     engine.close()
     model.close()

@@ -219,10 +219,10 @@ def test_batched_decode_matches_independent_sequences(gpu, lens):
         new = []
         for b in range(B):
             t_o, _, lg_o = oracles[b].forward([cur[b]])
-            e = H.mixed_err(engines[0].batch_logits(b), lg_o)
+            lg_g = engines[0].batch_logits(b)
+            e = H.mixed_err(lg_g, lg_o)
             worst = max(worst, e)
-            top = H.f16(lg_o)
-            assert nxt[b] == t_o or float(top.max() - top[nxt[b]]) <= 2 * H.TOL * 8, (step, b, nxt[b], t_o)
+            assert H.same_pick_or_near_tie(lg_g, lg_o, nxt[b], t_o), (step, b, nxt[b], t_o)
             new.append(t_o)
         cur = new
         assert [e.pos for e in engines] == [n + step + 1 for n in lens]
@@ -329,18 +329,16 @@ def test_llama3_8b_shapes_at_8k_context(gpu):
     e_l = H.mixed_err(lg_g, lg_o)
     say("8K context: hidden err", e_h, "all rows", e_all, "logits err", e_l, "tokens", tok_g, tok_o)
     assert e_all <= H.TOL and e_l <= H.TOL
-    top = H.f16(lg_o)
-    assert tok_g == tok_o or float(top.max() - top[tok_g]) <= 2 * H.TOL * 8
+    assert H.same_pick_or_near_tie(lg_g, lg_o, tok_g, tok_o)
     # decode at ctx 8192.. on the oracle's ids
     t = tok_o
     for step in range(6):
         t_g, h_g = eng.decode(int(t), want_hidden=True)
         t_o, h_o, lg_o = o.forward([int(t)], want_hidden=True)
         e = max(H.mixed_err(h_g, h_o), H.mixed_err(eng.logits(), lg_o))
-        top = H.f16(lg_o)
         say("  step", step, "err", e, t_g, t_o)
         assert e <= H.TOL
-        assert t_g == t_o or float(top.max() - top[t_g]) <= 2 * H.TOL * 8
+        assert H.same_pick_or_near_tie(eng.logits(), lg_o, t_g, t_o)
         t = t_o
     o.close()
     eng.close()
@@ -354,14 +352,22 @@ def _check_forced(r):
     assert max(r["forced_hidden_err"]) <= tol, r["forced_hidden_err"]
     assert max(r["forced_decode_hidden_err"]) <= tol, r["forced_decode_hidden_err"]
     assert max(r["forced_logits_err"]) <= tol, r["forced_logits_err"]
-    # greedy ids on identical context: equal, or the oracle's own logits of the two ids are closer
-    # than the logit tolerance allows to tell apart
-    for s, (a, b, gap) in enumerate(zip(r["tokens_oracle"], r["tokens_gpu_forced"], r["forced_gap_at_pick"])):
-        assert a == b or gap <= 2 * tol * 8, (s, a, b, gap)
-    # free running: the engine drifts from the oracle no further than a few times what reordering the
-    # oracle's own fp32 sums does (both compound through the same fp16 roundings)
-    for l, (free, floor) in enumerate(zip(r["free_hidden_err"], r["floor_hidden_err"])):
-        assert free <= tol + 4 * floor, (l, free, floor)
+    # greedy ids on identical context: equal, or the oracle holds the two ids closer together than
+    # the engine's measured logit error at exactly those two ids (no constant allowance)
+    for s, (a, b, gap, err) in enumerate(zip(r["tokens_oracle"], r["tokens_gpu_forced"],
+                                             r["forced_gap_at_pick"], r["forced_pick_err"])):
+        assert a == b or gap <= err, (s, a, b, gap, err)
+    # free running, anchored on exact arithmetic: per layer the engine is as close to ORC_FP32 (no
+    # intermediate rounding) as the reference's own rounding schedule (ORC_REF16) is.  Both the worst
+    # element and the root mean square over the layer; the additive term is one fp16 ulp of the
+    # tolerance scale so that layers whose error is a single flipped ulp do not decide the ratio.
+    for l in range(len(r["exact_err_hip"])):
+        assert r["exact_err_hip"][l] <= 1.5 * r["exact_err_ref16"][l] + 1e-3, (l, r["exact_err_hip"][l], r["exact_err_ref16"][l])
+        assert r["exact_rms_hip"][l] <= 1.5 * r["exact_rms_ref16"][l] + 1e-4, (l, r["exact_rms_hip"][l], r["exact_rms_ref16"][l])
+    assert r["exact_logits_err_hip"] <= 1.5 * r["exact_logits_err_ref16"] + 1e-3
+    # where the free-running ids part from the oracle's (if they do), the oracle's own logits of the
+    # two ids differ by less than the model tolerance of the logits
+    assert r["free_divergence_gap"] <= 2 * tol * (1 + r.get("free_divergence_logit_scale", 0.0)), r["free_divergence_gap"]
 
 
 def test_llama3_8b_full_depth_parity(gpu):
@@ -369,12 +375,15 @@ def test_llama3_8b_full_depth_parity(gpu):
     greedy steps, against the ORC_REF16 oracle.  Random-init LLaMA at this depth amplifies one-ulp fp16
     rounding differences from layer to layer, so the comparison is made three ways (see
     helpers.run_forced_parity): layer by layer on identical inputs (asserted to 2e-2), free running
-    (asserted against the drift of the oracle under a reversed summation order), and on the greedy ids."""
+    (the engine's distance from unrounded arithmetic, ORC_FP32, asserted to be no more than 1.5x that of
+    the reference's own rounding schedule), and on the greedy ids."""
     cfg = gpu.engine.config("8b", max_pos=128)
     say("8B full depth: generating weights, oracle forward ...")
     r = H.run_forced_parity(gpu, cfg, seed=2024, n_prompt=32, n_decode=32)
     say({k: (np.round(v, 4).tolist() if isinstance(v, list) and v and isinstance(v[0], float) else v)
          for k, v in r.items()})
+    say("8B full depth: free-running greedy ids identical to the oracle's for the first",
+        r["free_identical_prefix"], "of 32; oracle logit gap where they part:", r["free_divergence_gap"])
     _check_forced(r)
     assert sum(a == b for a, b in zip(r["tokens_oracle"], r["tokens_gpu_forced"])) >= 30
 
