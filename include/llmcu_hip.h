@@ -156,6 +156,18 @@ int llm_attn_decode(const uint16_t *q_dev, const uint16_t *k_cache_dev, const ui
                     uint16_t *out_dev, int ctx_host, const int32_t *ctx_dev, int n_heads,
                     int n_kv_heads, int head_dim, int max_pos, void *workspace_dev,
                     llm_stream_t stream);
+/* No counterpart in the reference: llm_attn_decode for callers that cannot allocate device memory
+ * (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  Same
+ * arguments without the workspace: the partial results and counters live in an array built into the
+ * library's device code (llm_attn_decode_noalloc_max_bytes() = 4 259 968 bytes on each GPU the
+ * library runs on, held until the process ends), whose device address llm_init looks up once per
+ * device.  Calls no hipMalloc/hipFree.  Limits: n_heads <= 32 and head_dim <= 128, otherwise
+ * LLM_ERR_INVALID.  All calls on one GPU share the array: calls that overlap on one GPU (two
+ * streams, two threads) race; serialise them or use llm_attn_decode with separate workspaces. */
+size_t llm_attn_decode_noalloc_max_bytes(void);
+int llm_attn_decode_noalloc(const uint16_t *q_dev, const uint16_t *k_cache_dev, const uint16_t *v_cache_dev,
+                            uint16_t *out_dev, int ctx_host, const int32_t *ctx_dev, int n_heads,
+                            int n_kv_heads, int head_dim, int max_pos, llm_stream_t stream);
 /* The decode step's form: takes the raw projection row qkv ([(Hq+2Hkv)*hd],
  * not rotated), applies RoPE for position pos = pos_host + (pos_dev ? *pos_dev : 0)
  * to Q and K, appends K and V to the caches at that position, and attends over

@@ -121,6 +121,8 @@ HIP_ABI = {
     "llm_norm_lmhead_argmax": (_i, [_vp, _vp, C.c_double, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp, _vp]),
     "llm_attn_decode_workspace_bytes": (_sz, [_i, _i]),
     "llm_attn_decode": (_i, [_vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _i, _vp, _vp]),
+    "llm_attn_decode_noalloc_max_bytes": (_sz, []),
+    "llm_attn_decode_noalloc": (_i, [_vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _i, _vp]),
     "llm_attn_prefill": (_i, [_vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp]),
     "llm_lmhead_workspace_bytes": (_sz, [_i]),
     "llm_lmhead_argmax": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp, _vp]),

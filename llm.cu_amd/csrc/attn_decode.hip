@@ -17,6 +17,7 @@
 // the final output is rounded.
 #include <cfloat>
 #include <cmath>
+#include <mutex>
 
 #include "common.hpp"
 
@@ -587,6 +588,66 @@ int llm_attn_decode(const uint16_t *q, const uint16_t *kc, const uint16_t *vc, u
     a.n_kv_heads = n_kv_heads;
     a.max_pos = max_pos;
     return dispatch_decode<false>(a, n_heads, head_dim, workspace, (hipStream_t)stream);
+}
+
+// ---- the same operation for callers that cannot allocate -------------------------------------
+// The partial results (acc, m, l per span) and the per-KV-head counters live in a file-scope device
+// array sized for 32 query heads of 128 dims (LLaMA3-8B): 4 259 968 bytes on every GPU the library
+// runs on, held until the process ends.  The array's name is only a host-side handle; the device
+// address is fetched per device with hipGetSymbolAddress and that pointer is what kernels get.
+#define AD_STATIC_MAX_HEADS 32
+#define AD_STATIC_MAX_HEAD_DIM 128
+#define AD_STATIC_BYTES \
+    (sizeof(float) * AD_STATIC_MAX_HEADS * AD_MAX_SPLITS * (AD_STATIC_MAX_HEAD_DIM + 2) + sizeof(int) * AD_STATIC_MAX_HEADS)
+static __device__ __align__(256) unsigned char scratch[AD_STATIC_BYTES];
+
+#define AD_MAX_DEVICES 64
+static void *g_scratch_ptr[AD_MAX_DEVICES];
+static std::mutex g_scratch_mutex;
+
+// Device address of this device's copy of the array (the current device must be `device`).
+static int scratch_for_device(int device, void **ptr) {
+    LLM_REQUIRE(device >= 0 && device < AD_MAX_DEVICES, "llm_attn_decode_noalloc: device %d out of range", device);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[device]) {
+        void *p = nullptr;
+        LLM_HIP_CHECK(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        LLM_REQUIRE(p != nullptr, "llm_attn_decode_noalloc: no device address for the scratch array");
+        g_scratch_ptr[device] = p;
+    }
+    *ptr = g_scratch_ptr[device];
+    return LLM_OK;
+}
+
+// Called by llm_init with the selected device current.
+int attn_decode_static_setup(int device) {
+    void *p;
+    return scratch_for_device(device, &p);
+}
+
+size_t llm_attn_decode_noalloc_max_bytes(void) { return AD_STATIC_BYTES; }
+
+int llm_attn_decode_noalloc(const uint16_t *q, const uint16_t *kc, const uint16_t *vc, uint16_t *out, int ctx_host,
+                            const int32_t *ctx_dev, int n_heads, int n_kv_heads, int head_dim, int max_pos,
+                            llm_stream_t stream) {
+    LLM_REQUIRE(n_heads > 0 && head_dim > 0, "llm_attn_decode_noalloc: heads %d, head_dim %d", n_heads, head_dim);
+    const size_t need = llm_attn_decode_workspace_bytes(n_heads, head_dim);
+    LLM_REQUIRE(n_heads <= AD_STATIC_MAX_HEADS && head_dim <= AD_STATIC_MAX_HEAD_DIM && need <= AD_STATIC_BYTES,
+                "llm_attn_decode_noalloc: %d heads of %d dims need %zu scratch bytes; the built-in scratch holds %zu "
+                "(at most %d heads of at most %d dims): use llm_attn_decode with a workspace",
+                n_heads, head_dim, need, (size_t)AD_STATIC_BYTES, AD_STATIC_MAX_HEADS, AD_STATIC_MAX_HEAD_DIM);
+    int device = 0;
+    LLM_HIP_CHECK(hipGetDevice(&device));
+    void *ws = nullptr;
+    int rc = scratch_for_device(device, &ws);
+    if (rc != LLM_OK) return rc;
+    // The array keeps what the last call left, and the counters sit behind the partial results at an
+    // offset that depends on (n_heads, head_dim): after a call with another shape that spot holds
+    // floats.  Clear this shape's counters with a fill kernel (safe under graph capture).
+    char *counters = (char *)ws + sizeof(float) * (size_t)n_heads * AD_MAX_SPLITS * (head_dim + 2);
+    rc = llm_fill_zero(counters, sizeof(int) * (size_t)n_heads, stream);
+    if (rc != LLM_OK) return rc;
+    return llm_attn_decode(q, kc, vc, out, ctx_host, ctx_dev, n_heads, n_kv_heads, head_dim, max_pos, ws, stream);
 }
 
 int llm_attn_decode_rope(const uint16_t *qkv, uint16_t *kc, uint16_t *vc, uint16_t *out, int pos_host,

@@ -22,6 +22,7 @@ __global__ void fill_zero_kernel(uint32_t *p, size_t n_words) {
 }
 
 int gemm_init_workspace(); // gemm.hip: split-K partial-sum buffer
+extern "C" int attn_decode_static_setup(int device); // attn_decode.hip: address of its built-in scratch
 
 extern "C" {
 
@@ -53,6 +54,8 @@ int llm_init(int device) {
         llm_set_error("device %d is %s; this library holds gfx950 code only", device, prop.gcnArchName);
         return LLM_ERR_NO_DEVICE;
     }
+    int rc = attn_decode_static_setup(device);
+    if (rc != LLM_OK) return rc;
     return gemm_init_workspace();
 }
 

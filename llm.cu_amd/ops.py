@@ -125,6 +125,17 @@ def attn_decode(q, kc, vc, ctx, n_heads, n_kv_heads, head_dim, repeats=1):
     return d_o.download()
 
 
+def attn_decode_noalloc(q, kc, vc, ctx, n_heads, n_kv_heads, head_dim):
+    """llm_attn_decode_noalloc: the library's built-in scratch instead of a workspace argument."""
+    q, kc, vc = _u16(q), _u16(kc), _u16(vc)
+    max_pos = kc.shape[1]
+    d_q, d_k, d_v = DevBuf.from_host(q), DevBuf.from_host(kc), DevBuf.from_host(vc)
+    d_o = DevBuf((n_heads * head_dim,), np.uint16)
+    check(lib().llm_attn_decode_noalloc(d_q.ptr, d_k.ptr, d_v.ptr, d_o.ptr, ctx, None, n_heads, n_kv_heads,
+                                        head_dim, max_pos, None))
+    return d_o.download()
+
+
 def attn_prefill(q, kc, vc, pos0, n_heads, n_kv_heads, head_dim):
     q, kc, vc = _u16(q), _u16(kc), _u16(vc)
     T = q.shape[0]
