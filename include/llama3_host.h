@@ -144,8 +144,15 @@ void free_tokenizer(Llama3Tokenizer *tokenizer, int decode_size);
 char *llama3_chat_prompt(const char *user_input);
 
 /* The reference fixes vocab 128256, temperature 0.7, top-k 50, top-p 0.9 at compile time
- * (inference.cu:24-29); init_cache_cfg() sets the vocabulary, this sets all four. */
+ * (inference.cu:24-29).  llama3_sampler_config() sets all four for the reference-named sampler
+ * functions above when they are called directly (one process-wide setting, as in the reference).
+ * inference() does not read that setting: every CudaCache carries its own (the vocabulary of its
+ * configuration, the reference's other three constants), changed with llama3_cache_sampler_config(). */
 void llama3_sampler_config(int vocab, float temperature, int top_k, float top_p);
+void llama3_cache_sampler_config(CudaCache *c, float temperature, int top_k, float top_p);
+/* sample_next_token() with the four settings as arguments: tensor is float[vocab] scratch, half_tensor
+ * the fp16 logits [vocab].  Reads and writes no process-wide setting. */
+int llama3_sample_with(int vocab, float temperature, int top_k, float top_p, float *tensor, llm_half *half_tensor);
 /* inference() returns the greedy id (0, default) or sample_next_token() of the logits as the
  * reference does (1). */
 void llama3_set_sampling(CudaCache *c, int on);

@@ -182,6 +182,8 @@ HOST_ABI = {
     "top_p_sampling": (_i, [_vp, C.c_float]),
     "llama3_sampler_config": (None, [_i, C.c_float, _i, C.c_float]),
     "llama3_set_sampling": (None, [_CP, _i]),
+    "llama3_cache_sampler_config": (None, [_CP, C.c_float, _i, C.c_float]),
+    "llama3_sample_with": (_i, [_i, C.c_float, _i, C.c_float, _vp, _vp]),
 }
 
 _lib = None

@@ -342,10 +342,10 @@ static int launch_prefill(const half_t *q, int ldq, const half_t *kc, const half
     dim3 grid(n_kv_heads, (n_qt + AP_QT - 1) / AP_QT);
     const size_t smem = sizeof(half_t) * 2 * ((size_t)AP_BKEY * (HD + 8) + (size_t)HD * (AP_BKEY + 8));
     auto kern = attn_prefill_kernel<HD, G, AP_QT>;
-    static bool attr_set = false;
-    if (!attr_set && smem > 48 * 1024) {
-        LLM_HIP_CHECK(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-        attr_set = true;
+    static std::atomic<uint64_t> attr_done{0};
+    if (smem > 48 * 1024) {
+        int rc = llm_ensure_max_smem((const void *)kern, smem, attr_done);
+        if (rc != LLM_OK) return rc;
     }
     kern<<<grid, dim3(G * AP_QT * 64), smem, s>>>(q, ldq, kc, vc, out, ldo, T, pos0, max_pos);
     LLM_LAUNCH_CHECK("attn_prefill_kernel");

@@ -3,6 +3,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "llmcu_hip.h"
 
 typedef _Float16 half_t;
@@ -45,6 +47,33 @@ void llm_set_error(const char *fmt, ...) __attribute__((format(printf, 1, 2)));
             return LLM_ERR_HIP;                                                     \
         }                                                                           \
     } while (0)
+
+// hipFuncSetAttribute(MaxDynamicSharedMemorySize) once per device for one kernel instantiation.
+// `done` is that instantiation's bit mask of devices already set; two threads racing on a fresh device
+// both set the same value, which is harmless.
+static inline int llm_ensure_max_smem(const void *kern, size_t smem, std::atomic<uint64_t> &done) {
+    int dev = 0;
+    LLM_HIP_CHECK(hipGetDevice(&dev));
+    const uint64_t bit = 1ull << (dev & 63);
+    if (done.load(std::memory_order_acquire) & bit) return LLM_OK;
+    LLM_HIP_CHECK(hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+    done.fetch_or(bit, std::memory_order_release);
+    return LLM_OK;
+}
+
+// Compute units of the current device (looked up once per device).
+static inline int llm_cu_count_cached(int *cus) {
+    static std::atomic<int> cache[64];
+    int dev = 0;
+    LLM_HIP_CHECK(hipGetDevice(&dev));
+    int n = cache[dev & 63].load(std::memory_order_relaxed);
+    if (n == 0) {
+        LLM_HIP_CHECK(hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev));
+        cache[dev & 63].store(n, std::memory_order_relaxed);
+    }
+    *cus = n;
+    return LLM_OK;
+}
 
 static inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 

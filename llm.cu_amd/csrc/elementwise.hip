@@ -96,9 +96,9 @@ __global__ __launch_bounds__(256) void add_residual_kernel(half_t *__restrict__ 
 // RMSNorm: one block per row (see rms_device.hpp for the summation order).
 // ---------------------------------------------------------------------------
 template <int THREADS>
-__global__ __launch_bounds__(THREADS) void rmsnorm_kernel(const half_t *__restrict__ x,
+__global__ __launch_bounds__(THREADS) void rmsnorm_kernel(const half_t *x, // may alias y
                                                           const half_t *__restrict__ gain,
-                                                          half_t *__restrict__ y, int d, double eps) {
+                                                          half_t *y, int d, double eps) {
     __shared__ float red[THREADS + 1];
     const size_t row = blockIdx.x;
     rms_normalise_row<THREADS>(x + row * d, gain, y + row * d, d, eps, red);

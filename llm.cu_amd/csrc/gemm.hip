@@ -14,7 +14,9 @@
 //   32x32x16: A lane l -> row l%32, k = 8*(l/32)..+7;  B lane l -> col l%32, same k;
 //             D lane l -> col l%32, rows 8*(i/4) + 4*(l/32) + i%4, i<16.
 #include <cmath>
+#include <mutex>
 #include <type_traits>
+#include <vector>
 
 #include "common.hpp"
 
@@ -37,8 +39,8 @@ template <bool SWIGLU>
 __global__ __launch_bounds__(SK_WAVES * 64) void skinny_kernel(const half_t *__restrict__ x, int ldx,
                                                                const half_t *__restrict__ w,
                                                                const half_t *__restrict__ w2,
-                                                               const half_t *__restrict__ res, int ldr,
-                                                               half_t *__restrict__ out, int ldo, int T,
+                                                               const half_t *res, int ldr, // may alias out
+                                                               half_t *out, int ldo, int T,
                                                                int N, int K) {
     __shared__ float red[SWIGLU ? 2 : 1][SK_WAVES][64][4];
     const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
@@ -301,18 +303,13 @@ static int skinny_dma_launch(const half_t *x, int ldx, const half_t *w, const ha
     static_assert(sizeof(half_t) * WAVES * (D + 1) * ((SWIGLU ? 2 : 1) + (XLDS ? 1 : 0)) * 16 * SKD_CHUNK <= 144 * 1024,
                   "ring does not fit beside the reduction buffers");
     auto kern = skinny_dma_kernel<SWIGLU, WAVES, D, XLDS>;
-    static bool attr_set = false;
-    if (!attr_set) {
-        LLM_HIP_CHECK(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-        attr_set = true;
-    }
+    static std::atomic<uint64_t> attr_done{0};
+    int rc = llm_ensure_max_smem((const void *)kern, smem, attr_done);
+    if (rc != LLM_OK) return rc;
     // the LDS tiles allow one workgroup per CU: as many workgroups as CUs, each walking over column tiles
-    static int cus = 0;
-    if (cus == 0) {
-        int dev = 0;
-        LLM_HIP_CHECK(hipGetDevice(&dev));
-        LLM_HIP_CHECK(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
-    }
+    int cus = 0;
+    rc = llm_cu_count_cached(&cus);
+    if (rc != LLM_OK) return rc;
     const int tiles = (N + 15) / 16;
     kern<<<dim3(tiles < cus ? tiles : cus), dim3(WAVES * 64), smem, s>>>(x, ldx, w, w2, res, ldr, out, ldo, T, N, K);
     LLM_LAUNCH_CHECK("skinny_dma_kernel");
@@ -334,8 +331,8 @@ template <int BM, int BN, int WGM, int WGN, int NB>
 __global__ __launch_bounds__(WGM *WGN * 64) void gemm_kernel(const half_t *__restrict__ x, int ldx,
                                                              const half_t *__restrict__ w,
                                                              const half_t *__restrict__ w2,
-                                                             const half_t *__restrict__ res, int ldr,
-                                                             half_t *__restrict__ out, int ldo, int T,
+                                                             const half_t *res, int ldr, // may alias out
+                                                             half_t *out, int ldo, int T,
                                                              int N, int K, int tiles_m, int tiles_n) {
     constexpr int THREADS = WGM * WGN * 64;
     constexpr int TM = BM / WGM, TN = BN / WGN; // wave tile
@@ -511,10 +508,10 @@ static int gemm_launch(const half_t *x, int ldx, const half_t *w, const half_t *
     const int tiles_m = (T + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
     const size_t smem = sizeof(half_t) * (2 * (size_t)BM * GEMM_LD + 2 * (size_t)NB * BN * GEMM_LD);
     auto kern = gemm_kernel<BM, BN, WGM, WGN, NB>;
-    static bool attr_set = false;
-    if (!attr_set && smem > 48 * 1024) {
-        LLM_HIP_CHECK(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-        attr_set = true;
+    static std::atomic<uint64_t> attr_done{0};
+    if (smem > 48 * 1024) {
+        int rc = llm_ensure_max_smem((const void *)kern, smem, attr_done);
+        if (rc != LLM_OK) return rc;
     }
     kern<<<dim3(tiles_m * tiles_n), dim3(WGM * WGN * 64), smem, s>>>(x, ldx, w, w2, res, ldr, out, ldo, T, N, K,
                                                                      tiles_m, tiles_n);
@@ -825,13 +822,54 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float *__restr
     *reinterpret_cast<half4_t *>(out + (size_t)m * ldo + n) = o;
 }
 
-// fp32 partial tiles of split-K launches; one buffer per process, allocated by llm_init
-static float *g_splitk_ws = nullptr;
+// fp32 partial tiles of split-K launches: one 64 MB buffer per (device, stream), so that launches on
+// different streams never share partial sums.  llm_init allocates the default stream's buffer; any
+// other stream gets its own at its first split-K launch (these run at 17..1024 rows, never inside a
+// captured decode step) and gives it back in llm_stream_destroy.  Without a buffer (allocation failed)
+// the launch runs unsplit.
 static const size_t SPLITK_WS_BYTES = (size_t)64 << 20;
+struct SplitkWs {
+    int device;
+    hipStream_t stream;
+    float *ptr;
+};
+static std::mutex g_splitk_mutex;
+static std::vector<SplitkWs> g_splitk_ws;
+
+static float *splitk_ws_for(hipStream_t s) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return nullptr;
+    std::lock_guard<std::mutex> lock(g_splitk_mutex);
+    for (const SplitkWs &e : g_splitk_ws)
+        if (e.device == dev && e.stream == s) return e.ptr;
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (s && hipStreamIsCapturing(s, &cap) == hipSuccess && cap != hipStreamCaptureStatusNone) return nullptr;
+    float *p = nullptr;
+    if (hipMalloc((void **)&p, SPLITK_WS_BYTES) != hipSuccess) {
+        (void)hipGetLastError();
+        return nullptr;
+    }
+    g_splitk_ws.push_back({dev, s, p});
+    return p;
+}
 
 int gemm_init_workspace() {
-    if (!g_splitk_ws) LLM_HIP_CHECK(hipMalloc((void **)&g_splitk_ws, SPLITK_WS_BYTES));
+    if (!splitk_ws_for(nullptr)) {
+        llm_set_error("llm_init: no memory for the split-K workspace");
+        return LLM_ERR_HIP;
+    }
     return LLM_OK;
+}
+
+// llm_stream_destroy: the stream's work has finished, its buffer goes back
+void gemm_release_workspace(hipStream_t s) {
+    std::lock_guard<std::mutex> lock(g_splitk_mutex);
+    for (size_t i = 0; i < g_splitk_ws.size(); ++i) {
+        if (g_splitk_ws[i].stream != s || s == nullptr) continue;
+        (void)hipFree(g_splitk_ws[i].ptr);
+        g_splitk_ws.erase(g_splitk_ws.begin() + (long)i);
+        --i;
+    }
 }
 
 template <int NB, int WGM, int WGN, int STAGES, bool PREF, int OCC, int FM = 2>
@@ -841,17 +879,17 @@ static int gemm_dma_launch(const half_t *x, int ldx, const half_t *w, const half
     const int tiles_m = (T + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
     const size_t smem = sizeof(half_t) * (size_t)STAGES * (BM + WGN * 128) * DMA_BK;
     auto kern = gemm_dma_kernel<NB, WGM, WGN, STAGES, PREF, OCC, FM>;
-    static bool attr_set = false;
-    if (!attr_set) {
-        LLM_HIP_CHECK(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-        attr_set = true;
-    }
+    static std::atomic<uint64_t> attr_done{0};
+    int rc = llm_ensure_max_smem((const void *)kern, smem, attr_done);
+    if (rc != LLM_OK) return rc;
+    float *ws = splits > 1 ? splitk_ws_for(s) : nullptr;
+    if (splits > 1 && !ws) splits = 1;
     if (splits > 1) {
         kern<<<dim3(tiles_m * tiles_n, splits), dim3(WGM * WGN * 64), smem, s>>>(x, ldx, w, w2, nullptr, 0, out, ldo, T, N, K,
-                                                                               tiles_m, tiles_n, g_splitk_ws, K / splits);
+                                                                               tiles_m, tiles_n, ws, K / splits);
         LLM_LAUNCH_CHECK("gemm_dma_kernel (split-K)");
         const size_t groups = (size_t)T * (N / 4);
-        splitk_reduce_kernel<NB><<<dim3((unsigned)((groups + 255) / 256)), dim3(256), 0, s>>>(g_splitk_ws, splits, T, N, res, ldr, out, ldo);
+        splitk_reduce_kernel<NB><<<dim3((unsigned)((groups + 255) / 256)), dim3(256), 0, s>>>(ws, splits, T, N, res, ldr, out, ldo);
         LLM_LAUNCH_CHECK("splitk_reduce_kernel");
         return LLM_OK;
     }
@@ -866,7 +904,7 @@ static int gemm_dma_launch(const half_t *x, int ldx, const half_t *w, const half
 static int pick_splits(long tiles, int T, int N, int K, int planes = 1) {
     int s = 1;
     while (s < 8 && tiles * s < 256 && K % (2 * s * DMA_BK) == 0 && K / (2 * s) >= 256 &&
-           (size_t)(2 * s) * planes * T * N * sizeof(float) <= SPLITK_WS_BYTES && g_splitk_ws)
+           (size_t)(2 * s) * planes * T * N * sizeof(float) <= SPLITK_WS_BYTES)
         s *= 2;
     return s;
 }

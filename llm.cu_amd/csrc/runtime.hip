@@ -21,7 +21,8 @@ __global__ void fill_zero_kernel(uint32_t *p, size_t n_words) {
     for (; i < n_words; i += stride) p[i] = 0u;
 }
 
-int gemm_init_workspace(); // gemm.hip: split-K partial-sum buffer
+int gemm_init_workspace(); // gemm.hip: split-K partial-sum buffer of the default stream
+void gemm_release_workspace(hipStream_t s); // gemm.hip: a stream's split-K buffer
 extern "C" int attn_decode_static_setup(int device); // attn_decode.hip: address of its built-in scratch
 
 extern "C" {
@@ -137,7 +138,11 @@ int llm_stream_create(llm_stream_t *stream) {
 }
 
 int llm_stream_destroy(llm_stream_t stream) {
-    if (stream) LLM_HIP_CHECK(hipStreamDestroy((hipStream_t)stream));
+    if (stream) {
+        LLM_HIP_CHECK(hipStreamSynchronize((hipStream_t)stream));
+        gemm_release_workspace((hipStream_t)stream);
+        LLM_HIP_CHECK(hipStreamDestroy((hipStream_t)stream));
+    }
     return LLM_OK;
 }
 

@@ -157,13 +157,22 @@ class Engine:
                               prompt.size, n_decode, out.ctypes.data_as(C.POINTER(C.c_int)), C.byref(st))
         return out, st
 
-    def inference(self, tokens):
-        """The reference's call: tokens[0] = n + 1, ids in tokens[1..n]."""
+    def inference(self, tokens, d_tokens=None):
+        """The reference's call: tokens[0] = n + 1, ids in tokens[1..n].  d_tokens: the device int
+        array of tokens_to_cuda (a capi.DevBuf of at least 2048 int32), or None."""
         n = len(tokens)
         arr = np.zeros(2049, np.int32)
         arr[0] = n + 1
         arr[1:n + 1] = tokens
-        return lib().inference(self.model.handle, None, None, arr.ctypes.data_as(C.POINTER(C.c_int)), self.cache)
+        dt = C.cast(d_tokens.ptr, C.POINTER(C.c_int)) if d_tokens is not None else None
+        return lib().inference(self.model.handle, None, dt, arr.ctypes.data_as(C.POINTER(C.c_int)), self.cache)
+
+    def host_logits(self):
+        """CudaCache.h_token_probdist: the fp16 logits inference() left on the host."""
+        return np.ctypeslib.as_array(self.cache.contents.h_token_probdist, shape=(self.cfg.vocab,)).copy()
+
+    def sampler_config(self, temperature, top_k, top_p):
+        lib().llama3_cache_sampler_config(self.cache, temperature, top_k, top_p)
 
     @staticmethod
     def decode_batch(engines, tokens):

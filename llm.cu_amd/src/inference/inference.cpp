@@ -22,12 +22,24 @@
 #include "llama3/llama3.h"
 #include "llama3_host.h"
 #include "llmcu_hip.h"
+#include "sampler.h"
 
 namespace {
 
 struct Engine {
     ModelConfig cfg;
+    const Llama3 *model = nullptr; // whose weight pointers the captured graphs hold
+    const void *model_slab = nullptr;
+    SamplerParams sampler;         // this cache's own settings (vocab = cfg.vocab)
     llm_stream_t stream = nullptr;
+    void *splitk_ws = nullptr;     // fp32 partial tiles of split-K projections issued on `stream`
+    size_t splitk_bytes = 0;
+    // pinned staging: [0] token in, [1] position in, [2] token out.  Reused by every step; safe because
+    // each step ends in a stream sync before the next one writes them.
+    int32_t *h_stage = nullptr;
+    // what the device holds after the last step: *d_pos == pos and d_tokens[pos] == dev_next (or -1)
+    bool dev_pos_valid = false;
+    int dev_next = -1;
     int qkv_dim = 0;
     // activations, sized for max_pos rows
     llm_half *x = nullptr, *xn = nullptr, *qkv = nullptr, *attn = nullptr, *ffn = nullptr;
@@ -113,6 +125,26 @@ void check_shapes(const Llama3 *m, const ModelConfig &c) {
     }
 }
 
+void drop_graph(Engine *e) {
+    for (int f = 0; f < 2; ++f) {
+        if (!e->graph[f]) continue;
+        llm_graph_destroy(e->graph[f]);
+        e->graph[f] = nullptr;
+    }
+}
+
+// The captured decode graphs hold the weight pointers of the model they were captured with.  A call
+// with another model (or the same struct after its weights were reloaded) is checked against the
+// configuration like the first one and the graphs are captured again.
+void bind_model(Engine *e, const Llama3 *m) {
+    const void *slab = m && m->embed_tokens ? (const void *)m->embed_tokens->d_fp16_tensor : nullptr;
+    if (m == e->model && slab == e->model_slab) return;
+    check_shapes(m, e->cfg);
+    drop_graph(e);
+    e->model = m;
+    e->model_slab = slab;
+}
+
 // Issues one pass over T rows on the engine's stream.  With dev_pos the row
 // position comes from *d_pos (T must be 1): that form is what gets captured.
 void issue_pass(Engine *e, const Llama3 *m, int T, int pos0, bool dev_pos, bool trace, bool inject = false) {
@@ -189,27 +221,21 @@ void issue_pass(Engine *e, const Llama3 *m, int T, int pos0, bool dev_pos, bool 
                  "llm_norm_lmhead_argmax");
 }
 
-void drop_graph(Engine *e) {
-    for (int f = 0; f < 2; ++f) {
-        if (!e->graph[f]) continue;
-        llm_graph_destroy(e->graph[f]);
-        e->graph[f] = nullptr;
-    }
-}
-
 // Appends n host tokens at e->pos with one multi-row pass.  Leaves
 // d_pos = pos + n and d_tokens[pos + n] = the greedy next token.
-int run_pass(Engine *e, const Llama3 *m, const int *tokens, int n) {
+// logits_host (may be null): pinned host memory that receives the fp16 logits before the pass's one sync.
+int run_pass(Engine *e, const Llama3 *m, const int *tokens, int n, llm_half *logits_host = nullptr) {
     const ModelConfig &c = e->cfg;
+    bind_model(e, m);
     if (n < 1) llama3_fail("a pass needs at least one token");
     if (e->pos + n > c.max_pos) llama3_fail("sequence of %d tokens exceeds max_pos %d", e->pos + n, c.max_pos);
     for (int i = 0; i < n; ++i)
         if (tokens[i] < 0 || tokens[i] >= c.vocab) llama3_fail("token id %d outside the vocabulary", tokens[i]);
     llm_stream_t s = e->stream;
     llama3_check(llm_memcpy_h2d(e->d_tokens + e->pos, tokens, sizeof(int) * (size_t)n, s), "H2D tokens");
-    const int32_t last = e->pos + n - 1;
-    llama3_check(llm_memcpy_h2d(e->d_pos, &last, sizeof(int32_t), s), "H2D position");
-    llama3_check(llm_stream_sync(s), "stream sync"); // `last` is a stack variable
+    e->h_stage[1] = e->pos + n - 1;
+    llama3_check(llm_memcpy_h2d(e->d_pos, &e->h_stage[1], sizeof(int32_t), s), "H2D position");
+    llama3_check(llm_stream_sync(s), "stream sync"); // `tokens` is the caller's (pageable) memory
     const bool trace = e->trace_host != nullptr;
     if (trace) {
         size_t need = (size_t)c.n_layers * n * c.d_model;
@@ -231,17 +257,21 @@ int run_pass(Engine *e, const Llama3 *m, const int *tokens, int n) {
     }
     e->long_attn = n == 1 && e->pos >= LONG_ATTN_FROM; // single rows go through the decode kernels
     issue_pass(e, m, n, e->pos, false, trace, inject);
-    int32_t tok = -1;
-    llama3_check(llm_memcpy_d2h(&tok, e->d_token, sizeof(int32_t), s), "D2H token");
+    llama3_check(llm_memcpy_d2h(&e->h_stage[2], e->d_token, sizeof(int32_t), s), "D2H token");
     if (trace)
         llama3_check(llm_memcpy_d2h(e->trace_host, e->trace_dev, sizeof(llm_half) * (size_t)c.n_layers * n * c.d_model, s),
                      "D2H trace");
+    if (logits_host)
+        llama3_check(llm_memcpy_d2h(logits_host, e->logits, sizeof(llm_half) * (size_t)c.vocab, s), "D2H logits");
     llama3_check(llm_stream_sync(s), "stream sync");
     e->trace_host = nullptr;
     e->inject_host = nullptr;
     e->tokens.insert(e->tokens.end(), tokens, tokens + n);
     e->pos += n;
-    return (int)tok;
+    // the pass left *d_pos == pos and its pick in d_tokens[pos]
+    e->dev_pos_valid = true;
+    e->dev_next = e->h_stage[2];
+    return (int)e->h_stage[2];
 }
 
 // One decode step from device state (d_tokens[*d_pos] in, next token out).
@@ -266,6 +296,37 @@ void launch_decode_step(Engine *e, const Llama3 *m, int pos) {
     }
 }
 
+// One cached decode step with a single host round trip: the token id and the position go up only when
+// the device does not already hold them (after a greedy step it does: the argmax kernel stored its pick
+// at d_tokens[pos] and advanced *d_pos), the result (and, when asked for, the logits) come back through
+// pinned memory, one stream sync at the end.
+int step_one(Engine *e, const Llama3 *m, int token, llm_half *logits_host) {
+    if (e->trace_host || e->inject_host) return run_pass(e, m, &token, 1, logits_host);
+    const ModelConfig &c = e->cfg;
+    bind_model(e, m);
+    if (e->pos + 1 > c.max_pos) llama3_fail("sequence of %d tokens exceeds max_pos %d", e->pos + 1, c.max_pos);
+    if (token < 0 || token >= c.vocab) llama3_fail("token id %d outside the vocabulary", token);
+    llm_stream_t s = e->stream;
+    if (!e->dev_pos_valid || e->dev_next != token) {
+        e->h_stage[0] = token;
+        llama3_check(llm_memcpy_h2d(e->d_tokens + e->pos, &e->h_stage[0], sizeof(int32_t), s), "H2D token");
+    }
+    if (!e->dev_pos_valid) {
+        e->h_stage[1] = e->pos;
+        llama3_check(llm_memcpy_h2d(e->d_pos, &e->h_stage[1], sizeof(int32_t), s), "H2D position");
+    }
+    launch_decode_step(e, m, e->pos);
+    llama3_check(llm_memcpy_d2h(&e->h_stage[2], e->d_token, sizeof(int32_t), s), "D2H token");
+    if (logits_host)
+        llama3_check(llm_memcpy_d2h(logits_host, e->logits, sizeof(llm_half) * (size_t)c.vocab, s), "D2H logits");
+    llama3_check(llm_stream_sync(s), "stream sync");
+    e->tokens.push_back(token);
+    e->pos += 1;
+    e->dev_pos_valid = true;
+    e->dev_next = e->h_stage[2];
+    return (int)e->h_stage[2];
+}
+
 } // namespace
 
 // ---------------------------------------------------------------------------
@@ -276,6 +337,9 @@ extern "C" CudaCache *init_cache_cfg(Llama3 *m, const ModelConfig *cfg) {
     check_shapes(m, c);
     Engine *e = new Engine;
     e->cfg = c;
+    e->model = m;
+    e->model_slab = m->embed_tokens->d_fp16_tensor;
+    e->sampler.vocab = c.vocab; // temperature 0.7, top-k 50, top-p 0.9 as in inference.cu:27-29
     const int d = c.d_model, qd = c.n_heads * c.head_dim, kvd = c.n_kv_heads * c.head_dim;
     e->qkv_dim = qd + 2 * kvd;
     const size_t R = (size_t)c.max_pos;
@@ -309,15 +373,23 @@ extern "C" CudaCache *init_cache_cfg(Llama3 *m, const ModelConfig *cfg) {
     llama3_check(llm_fill_zero(e->ws_attn, wa, e->stream), "zero attention workspace");
     llama3_check(llm_malloc(&e->ws_lm, llm_lmhead_workspace_bytes(c.vocab)), "llm_malloc(lm head workspace)");
     for (auto &ev : e->ev) llama3_check(llm_event_create(&ev), "llm_event_create");
+    {
+        void *hs = nullptr;
+        llama3_check(llm_malloc_host(&hs, sizeof(int32_t) * 8), "llm_malloc_host(staging)");
+        e->h_stage = (int32_t *)hs;
+    }
     llama3_check(llm_stream_sync(e->stream), "stream sync");
 
     CudaCache *C = (CudaCache *)calloc(1, sizeof(CudaCache));
     if (!C) llama3_fail("Memory allocation failed for CudaCache");
     C->d_feedforward_cache_upgate = e->ffn;
     C->d_token_probdist = e->logits;
-    C->h_token_probdist = (llm_half *)malloc(sizeof(llm_half) * (size_t)c.vocab);
+    // pinned, so that the logits of a step come back asynchronously behind its token id
+    void *hp = nullptr;
+    llama3_check(llm_malloc_host(&hp, sizeof(llm_half) * (size_t)c.vocab), "llm_malloc_host(h_token_probdist)");
+    C->h_token_probdist = (llm_half *)hp;
     C->f_token_probdist = (float *)malloc(sizeof(float) * (size_t)c.vocab);
-    llama3_sampler_config(c.vocab, 0.7f, 50, 0.9f); // inference.cu:27-29
+    if (!C->f_token_probdist) llama3_fail("Memory allocation failed for f_token_probdist");
     C->engine = e;
     return C;
 }
@@ -350,9 +422,10 @@ extern "C" void free_cache(CudaCache *C) {
         for (void *b : bufs) llm_free(b);
         for (auto ev : e->ev) llm_event_destroy(ev);
         llm_stream_destroy(e->stream);
+        llm_free_host(e->h_stage);
         delete e;
     }
-    free(C->h_token_probdist);
+    llm_free_host(C->h_token_probdist);
     free(C->f_token_probdist);
     free(C);
 }
@@ -379,6 +452,8 @@ extern "C" void llama3_cache_reset(CudaCache *C) {
     Engine *e = eng(C);
     e->pos = 0;
     e->tokens.clear();
+    e->dev_pos_valid = false;
+    e->dev_next = -1;
 }
 
 extern "C" int llama3_cache_pos(const CudaCache *C) { return eng(C)->pos; }
@@ -387,30 +462,13 @@ extern "C" int llama3_prefill(Llama3 *m, CudaCache *C, const int *tokens, int n)
     return run_pass(eng(C), m, tokens, n);
 }
 
-extern "C" int llama3_decode(Llama3 *m, CudaCache *C, int token) {
-    Engine *e = eng(C);
-    if (e->trace_host || e->inject_host) return run_pass(e, m, &token, 1);
-    const ModelConfig &c = e->cfg;
-    if (e->pos + 1 > c.max_pos) llama3_fail("sequence of %d tokens exceeds max_pos %d", e->pos + 1, c.max_pos);
-    if (token < 0 || token >= c.vocab) llama3_fail("token id %d outside the vocabulary", token);
-    llm_stream_t s = e->stream;
-    const int32_t p = e->pos, t = token;
-    llama3_check(llm_memcpy_h2d(e->d_tokens + e->pos, &t, sizeof(int32_t), s), "H2D token");
-    llama3_check(llm_memcpy_h2d(e->d_pos, &p, sizeof(int32_t), s), "H2D position");
-    llama3_check(llm_stream_sync(s), "stream sync");
-    launch_decode_step(e, m, e->pos);
-    int32_t tok = -1;
-    llama3_check(llm_memcpy_d2h(&tok, e->d_token, sizeof(int32_t), s), "D2H token");
-    llama3_check(llm_stream_sync(s), "stream sync");
-    e->tokens.push_back(token);
-    e->pos += 1;
-    return (int)tok;
-}
+extern "C" int llama3_decode(Llama3 *m, CudaCache *C, int token) { return step_one(eng(C), m, token, nullptr); }
 
 extern "C" int llama3_generate(Llama3 *m, CudaCache *C, const int *prompt, int n_prompt, int n_decode,
                                int *out_tokens, GenStats *stats) {
     Engine *e = eng(C);
     const ModelConfig &c = e->cfg;
+    bind_model(e, m);
     if (n_decode < 1) llama3_fail("llama3_generate: n_decode must be at least 1");
     if (e->pos + n_prompt + n_decode - 1 > c.max_pos)
         llama3_fail("prompt %d + %d decode steps exceed max_pos %d", e->pos + n_prompt, n_decode - 1, c.max_pos);
@@ -439,6 +497,8 @@ extern "C" int llama3_generate(Llama3 *m, CudaCache *C, const int *prompt, int n
     // host mirror: the decode steps consumed out_tokens[0..n_decode-2]
     for (int i = 0; i + 1 < n_decode; ++i) e->tokens.push_back(out_tokens[i]);
     e->pos += n_decode - 1;
+    e->dev_pos_valid = true; // every replayed step advanced *d_pos and stored its pick at d_tokens[pos]
+    e->dev_next = out_tokens[n_decode - 1];
     if (stats) {
         float a = 0.f, b = 0.f;
         llm_event_elapsed_ms(e->ev[0], e->ev[1], &a);
@@ -462,6 +522,7 @@ extern "C" void llama3_decode_batch(Llama3 *m, CudaCache *const *caches, const i
     if (batch < 1 || batch > 16) llama3_fail("llama3_decode_batch: batch %d (1..16)", batch);
     Engine *e0 = eng(caches[0]);
     const ModelConfig &c = e0->cfg;
+    bind_model(e0, m);
     const int d = c.d_model, hd = c.head_dim, Hq = c.n_heads, Hkv = c.n_kv_heads, F = c.ffn_dim;
     const int qd = Hq * hd, kvd = Hkv * hd, QKV = e0->qkv_dim;
     llm_stream_t s = e0->stream;
@@ -531,6 +592,7 @@ extern "C" void llama3_decode_batch(Llama3 *m, CudaCache *const *caches, const i
         next_tokens[b] = (int)out[b];
         es[b]->tokens.push_back(tokens[b]);
         es[b]->pos += 1;
+        es[b]->dev_pos_valid = false; // the batched step keeps no per-cache position on the device
     }
 }
 
@@ -570,17 +632,33 @@ extern "C" int inference(Llama3 *m, Tensor *X, int *d_tokens, int *h_tokens, Cud
     const int n = h_tokens[0] - 1;
     const int *ids = h_tokens + 1;
     if (n < 1) llama3_fail("inference: empty token list");
-    if (d_tokens) // the reference's H2D of the whole token array (inference.cu:150)
-        llama3_check(llm_memcpy_h2d(d_tokens, h_tokens, sizeof(int) * (size_t)(n + 1 < 2048 ? n + 1 : 2048), nullptr),
-                     "H2D tokens");
     bool extend = n > e->pos;
     for (int i = 0; extend && i < e->pos; ++i) extend = ids[i] == e->tokens[i];
     if (!extend) llama3_cache_reset(C);
+    if (d_tokens) {
+        // the reference's H2D of the token array (inference.cu:150); nothing here reads it back, so only
+        // the entries that changed since the last call go up (the count and the new ids), in stream order
+        const int first_new = e->pos + 1, last = n < 2047 ? n : 2047;
+        llama3_check(llm_memcpy_h2d(d_tokens, h_tokens, sizeof(int), e->stream), "H2D token count");
+        if (last >= first_new)
+            llama3_check(llm_memcpy_h2d(d_tokens + first_new, h_tokens + first_new,
+                                        sizeof(int) * (size_t)(last - first_new + 1), e->stream),
+                         "H2D tokens");
+    }
     const int fresh = n - e->pos;
-    int tok = fresh == 1 ? llama3_decode(m, C, ids[n - 1]) : llama3_prefill(m, C, ids + e->pos, fresh);
-    llama3_read_logits(C, C->h_token_probdist);
-    if (e->sampling) tok = sample_next_token(C->f_token_probdist, C->h_token_probdist); // inference.cu:1028
+    // h_token_probdist holds the step's logits on return, as after the reference's compute_lm_head
+    // (inference.cu:1021-1026); they travel behind the token id in the same stream, one sync per call
+    int tok = fresh == 1 ? step_one(e, m, ids[n - 1], C->h_token_probdist)
+                         : run_pass(e, m, ids + e->pos, fresh, C->h_token_probdist);
+    if (e->sampling) tok = sampler_draw(e->sampler, C->f_token_probdist, C->h_token_probdist); // inference.cu:1028
     return tok;
 }
 
 extern "C" void llama3_set_sampling(CudaCache *C, int on) { eng(C)->sampling = on != 0; }
+
+extern "C" void llama3_cache_sampler_config(CudaCache *C, float temperature, int top_k, float top_p) {
+    Engine *e = eng(C);
+    e->sampler.temperature = temperature;
+    e->sampler.top_k = top_k;
+    e->sampler.top_p = top_p;
+}

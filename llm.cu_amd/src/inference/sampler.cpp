@@ -11,11 +11,11 @@
 
 #include "../common/fail.h"
 #include "llama3_host.h"
+#include "sampler.h"
 
-static int g_vocab = 128256;           // VOCAB_SIZE, inference.cu:24
-static float g_temperature = 0.7f;     // TEMPERATURE, inference.cu:27
-static int g_top_k = 50;               // TOP_K, inference.cu:28
-static float g_top_p = 0.9f;           // TOP_P, inference.cu:29
+// Settings of the reference-named entry points below, which take no settings argument (the reference
+// fixes them at compile time).  A CudaCache carries its own SamplerParams: inference() never reads these.
+static SamplerParams g_params; // VOCAB_SIZE, TEMPERATURE, TOP_K, TOP_P of inference.cu:24-29
 
 // __half2float: exact widening of an fp16 bit pattern
 static float half_to_float(llm_half h) {
@@ -40,47 +40,31 @@ static float half_to_float(llm_half h) {
     return f;
 }
 
-extern "C" {
-
-void llama3_sampler_config(int vocab, float temperature, int top_k, float top_p) {
-    if (vocab < 1) llama3_fail("llama3_sampler_config: vocab must be positive");
-    g_vocab = vocab;
-    g_temperature = temperature;
-    g_top_k = top_k;
-    g_top_p = top_p;
-}
-
-// inference.cu:1074-1084
-int _compare_desc(const void *a, const void *b) {
-    const ProbIndex *pa = (const ProbIndex *)a, *pb = (const ProbIndex *)b;
-    if (pa->probability < pb->probability) return 1;
-    if (pa->probability > pb->probability) return -1;
-    return 0;
-}
+extern "C" int _compare_desc(const void *a, const void *b);
 
 // inference.cu:1043-1072
-ProbIndex *temperature_softmax(float *tensor, llm_half *half_tensor, float temperature) {
-    ProbIndex *arr = (ProbIndex *)malloc((size_t)g_vocab * sizeof(ProbIndex));
+static ProbIndex *softmax_sorted(int vocab, float *tensor, const llm_half *half_tensor, float temperature) {
+    ProbIndex *arr = (ProbIndex *)malloc((size_t)vocab * sizeof(ProbIndex));
     if (!arr) llama3_fail("temperature_softmax: out of memory");
     float cumsum = 0.0f;
-    for (int i = 0; i < g_vocab; ++i) {
+    for (int i = 0; i < vocab; ++i) {
         const float scaled = half_to_float(half_tensor[i]) / temperature;
         tensor[i] = expf(scaled);
         cumsum += tensor[i];
     }
-    for (int i = 0; i < g_vocab; ++i) {
+    for (int i = 0; i < vocab; ++i) {
         tensor[i] /= cumsum;
         arr[i].probability = tensor[i];
         arr[i].index = i;
     }
-    qsort(arr, (size_t)g_vocab, sizeof(ProbIndex), _compare_desc);
+    qsort(arr, (size_t)vocab, sizeof(ProbIndex), _compare_desc);
     return arr;
 }
 
 // inference.cu:1086-1113
-int top_k_sampling(ProbIndex *arr, int k) {
-    if (k <= 0) return arr[rand() % g_vocab].index;
-    if (k > g_vocab) k = g_vocab;
+static int top_k_pick(int vocab, ProbIndex *arr, int k) {
+    if (k <= 0) return arr[rand() % vocab].index;
+    if (k > vocab) k = vocab;
     float sum = 0.0f;
     for (int i = 0; i < k; ++i) sum += arr[i].probability;
     for (int i = 0; i < k; ++i) arr[i].probability /= sum;
@@ -93,18 +77,18 @@ int top_k_sampling(ProbIndex *arr, int k) {
     return arr[0].index;
 }
 
-// inference.cu:1115-1161
-int top_p_sampling(ProbIndex *arr, float p) {
-    if (p <= 0.0f) return arr[rand() % g_vocab].index;
+// inference.cu:1115-1161.  n: entries of arr that exist (the whole vocabulary in the reference's flow).
+static int top_p_pick(int vocab, ProbIndex *arr, int n, float p) {
+    if (p <= 0.0f) return arr[rand() % vocab].index;
     if (p > 1.0f) p = 1.0f;
     float cumulative = 0.0f;
     int cutoff = 0;
-    for (; cutoff < g_vocab; ++cutoff) {
+    for (; cutoff < n; ++cutoff) {
         cumulative += arr[cutoff].probability;
         if (cumulative >= p) break;
     }
     const float sum = cumulative;
-    if (cutoff >= g_vocab) cutoff = g_vocab - 1;
+    if (cutoff >= n) cutoff = n - 1;
     for (int i = 0; i <= cutoff; ++i) arr[i].probability /= sum;
     const float r = (float)rand() / (float)RAND_MAX;
     cumulative = 0.0f;
@@ -115,29 +99,27 @@ int top_p_sampling(ProbIndex *arr, float p) {
     return arr[0].index;
 }
 
-// inference.cu:1030-1041, call for call (a full qsort of the vocabulary per token: ~10 ms at 128256)
-int sample_next_token_reference(float *tensor, llm_half *half_tensor) {
-    ProbIndex *arr = temperature_softmax(tensor, half_tensor, g_temperature);
-    int selected = top_k_sampling(arr, g_top_k);
-    selected = top_p_sampling(arr, g_top_p);
+int sampler_draw_reference(const SamplerParams &sp, float *tensor, const llm_half *half_tensor) {
+    ProbIndex *arr = softmax_sorted(sp.vocab, tensor, half_tensor, sp.temperature);
+    int selected = top_k_pick(sp.vocab, arr, sp.top_k);
+    selected = top_p_pick(sp.vocab, arr, sp.vocab, sp.top_p);
     free(arr);
     return selected;
 }
 
-// Same result without sorting the vocabulary.  After top_k_sampling() has renormalised the first k
-// entries they sum to 1 up to rounding, so for top_p below that sum top_p_sampling() never looks past
+// Same result without sorting the vocabulary.  After the top-k pass has renormalised the first k
+// entries they sum to 1 up to rounding, so for top_p below that sum the top-p pass never looks past
 // entry k-1: only the k largest probabilities, in the order qsort leaves them, matter.  glibc's qsort
 // is a merge sort (stable) whenever it can allocate its buffer, so equal probabilities stay in index
 // order; partial_sort with the index as second key reproduces that head exactly.  Falls back to the
 // full path for settings where the tail of the array is reachable.
-int sample_next_token(float *tensor, llm_half *half_tensor) {
-    const int k = g_top_k;
-    if (k <= 0 || k >= g_vocab || !(g_top_p > 0.0f) || g_top_p > 0.99f)
-        return sample_next_token_reference(tensor, half_tensor);
+int sampler_draw(const SamplerParams &sp, float *tensor, const llm_half *half_tensor) {
+    const int k = sp.top_k, vocab = sp.vocab;
+    if (k <= 0 || k >= vocab || !(sp.top_p > 0.0f) || sp.top_p > 0.99f)
+        return sampler_draw_reference(sp, tensor, half_tensor);
     // the exponentials are independent (any thread gives the same bits); their sum is taken afterwards in
     // index order, as the reference's single loop does
-    const int vocab = g_vocab;
-    const float temperature = g_temperature;
+    const float temperature = sp.temperature;
 #pragma omp parallel for schedule(static)
     for (int i = 0; i < vocab; ++i) tensor[i] = expf(half_to_float(half_tensor[i]) / temperature);
     float cumsum = 0.0f;
@@ -145,17 +127,17 @@ int sample_next_token(float *tensor, llm_half *half_tensor) {
 #pragma omp parallel for schedule(static)
     for (int i = 0; i < vocab; ++i) tensor[i] /= cumsum;
     // NaN probabilities (exp overflow) defeat every comparison: let the reference path decide
-    if (!(cumsum < INFINITY) || !(cumsum > 0.0f)) return sample_next_token_reference(tensor, half_tensor);
+    if (!(cumsum < INFINITY) || !(cumsum > 0.0f)) return sampler_draw_reference(sp, tensor, half_tensor);
     // k largest by (probability desc, index asc): threshold pass, then a sort of the few survivors
-    ProbIndex *head = (ProbIndex *)malloc((size_t)(2 * k + 64) * sizeof(ProbIndex));
+    const int cap = 2 * k + 64;
+    ProbIndex *head = (ProbIndex *)malloc((size_t)cap * sizeof(ProbIndex));
     if (!head) llama3_fail("sample_next_token: out of memory");
     int n = 0;
-    const int cap = 2 * k + 64;
     float floor_p = -1.0f; // entries below the current k-th best cannot enter the head
     auto better = [](const ProbIndex &a, const ProbIndex &b) {
         return a.probability > b.probability || (a.probability == b.probability && a.index < b.index);
     };
-    for (int i = 0; i < g_vocab; ++i) {
+    for (int i = 0; i < vocab; ++i) {
         const float p = tensor[i];
         if (p < floor_p) continue; // ties with the floor come later in index order only if p == floor: keep them
         head[n].probability = p;
@@ -172,10 +154,57 @@ int sample_next_token(float *tensor, llm_half *half_tensor) {
     } else {
         std::sort(head, head + n, better);
     }
-    int selected = top_k_sampling(head, k);
-    selected = top_p_sampling(head, g_top_p);
+    int selected = top_k_pick(vocab, head, k);
+    selected = top_p_pick(vocab, head, k, sp.top_p);
     free(head);
     return selected;
 }
+
+extern "C" {
+
+void llama3_sampler_config(int vocab, float temperature, int top_k, float top_p) {
+    if (vocab < 1) llama3_fail("llama3_sampler_config: vocab must be positive");
+    g_params.vocab = vocab;
+    g_params.temperature = temperature;
+    g_params.top_k = top_k;
+    g_params.top_p = top_p;
+}
+
+// inference.cu:1074-1084
+int _compare_desc(const void *a, const void *b) {
+    const ProbIndex *pa = (const ProbIndex *)a, *pb = (const ProbIndex *)b;
+    if (pa->probability < pb->probability) return 1;
+    if (pa->probability > pb->probability) return -1;
+    return 0;
+}
+
+// The sampler with its settings as arguments (no process-wide state is read or written).
+int llama3_sample_with(int vocab, float temperature, int top_k, float top_p, float *tensor, llm_half *half_tensor) {
+    if (vocab < 1) llama3_fail("llama3_sample_with: vocab must be positive");
+    SamplerParams sp;
+    sp.vocab = vocab;
+    sp.temperature = temperature;
+    sp.top_k = top_k;
+    sp.top_p = top_p;
+    return sampler_draw(sp, tensor, half_tensor);
+}
+
+// inference.cu:1043-1072
+ProbIndex *temperature_softmax(float *tensor, llm_half *half_tensor, float temperature) {
+    return softmax_sorted(g_params.vocab, tensor, half_tensor, temperature);
+}
+
+// inference.cu:1086-1113
+int top_k_sampling(ProbIndex *arr, int k) { return top_k_pick(g_params.vocab, arr, k); }
+
+// inference.cu:1115-1161
+int top_p_sampling(ProbIndex *arr, float p) { return top_p_pick(g_params.vocab, arr, g_params.vocab, p); }
+
+// inference.cu:1030-1041, call for call (a full qsort of the vocabulary per token: ~10 ms at 128256)
+int sample_next_token_reference(float *tensor, llm_half *half_tensor) {
+    return sampler_draw_reference(g_params, tensor, half_tensor);
+}
+
+int sample_next_token(float *tensor, llm_half *half_tensor) { return sampler_draw(g_params, tensor, half_tensor); }
 
 } // extern "C"

@@ -15,7 +15,10 @@
 #include "llama3_host.h"
 #include "safetensor/json.h"
 
-static int g_decode_size = 128256;
+// Size of the decode table that the reference-named _build_decoder() checks ids against (its signature
+// carries no size).  Per thread, set by the load that is running on that thread; loads on different
+// threads do not see each other's value.
+static thread_local int g_decode_size = 128256;
 
 extern "C" {
 
@@ -104,9 +107,14 @@ void _build_trie(TrieNode *root, char *token_string, int token_int) {
 }
 
 // tokenizer.cu:334-343
+static void build_decoder_entry(char **decoder, int decode_size, char *token_string, int token_int);
 void _build_decoder(char **decoder, char *token_string, int token_int) {
-    if (token_int < 0 || token_int >= g_decode_size)
-        llama3_fail("token id %d is outside the decode table of %d entries", token_int, g_decode_size);
+    build_decoder_entry(decoder, g_decode_size, token_string, token_int);
+}
+
+static void build_decoder_entry(char **decoder, int decode_size, char *token_string, int token_int) {
+    if (token_int < 0 || token_int >= decode_size)
+        llama3_fail("token id %d is outside the decode table of %d entries", token_int, decode_size);
     free(decoder[token_int]);
     size_t length = strlen(token_string) + 1;
     decoder[token_int] = (char *)malloc(length);
@@ -139,7 +147,7 @@ Llama3Tokenizer *load_tokenizer_from(const char *filename, int decode_size) {
     for (const auto &kv : vocab->obj) {
         std::string s = kv.first;
         _build_trie(tok->root, &s[0], (int)kv.second.num);
-        _build_decoder(tok->decode, &s[0], (int)kv.second.num);
+        build_decoder_entry(tok->decode, decode_size, &s[0], (int)kv.second.num);
     }
     if (added->kind == minijson::Value::Array) {
         for (const minijson::Value &e : added->arr) {
@@ -147,7 +155,7 @@ Llama3Tokenizer *load_tokenizer_from(const char *filename, int decode_size) {
             if (id == nullptr || content == nullptr) continue;
             std::string s = content->str;
             _build_trie(tok->root, &s[0], (int)id->num);
-            _build_decoder(tok->decode, &s[0], (int)id->num);
+            build_decoder_entry(tok->decode, decode_size, &s[0], (int)id->num);
         }
     }
     return tok;

@@ -98,6 +98,83 @@ def test_reference_shaped_inference_call(gpu):
     model.close()
 
 
+def test_inference_call_leaves_logits_on_the_host_and_mirrors_d_tokens(gpu):
+    """After inference() returns, CudaCache.h_token_probdist holds the step's fp16 logits (as after the
+    reference's compute_lm_head, inference.cu:1021-1026) and the caller's d_tokens array holds the
+    token list; the greedy id is the argmax of exactly those logits."""
+    cfg, model, eng = _tiny_engine(gpu)
+    d_tokens = gpu.capi.DevBuf((2048,), np.int32)
+    d_tokens.zero()
+    seq = [int(t) for t in gpu.engine.seeded_tokens(9, 10, cfg.vocab)]
+    for step in range(5):
+        tok = eng.inference(seq, d_tokens)
+        lg = eng.host_logits()
+        assert np.array_equal(lg, eng.logits())
+        assert tok == orc.argmax_f16(lg)
+        mirror = d_tokens.download()
+        assert mirror[0] == len(seq) + 1 and list(mirror[1:len(seq) + 1]) == seq
+        # a caller that does not follow the greedy id (a sampler): the step must use the caller's id
+        seq.append(tok if step % 2 == 0 else (tok + 1) % cfg.vocab)
+    # same sequence through the stepwise API on a fresh cache
+    eng2 = gpu.engine.Engine(model, cfg, use_graph=False)
+    t2, _ = eng2.prefill(np.array(seq[:-1], np.int32))
+    assert t2 == tok
+    eng.close()
+    eng2.close()
+    model.close()
+
+
+def test_two_caches_with_different_vocabularies_sample_independently(gpu):
+    """Sampler settings live in the cache: two live caches of different vocabulary sizes, inference() with
+    the reference's sampler on both, interleaved; each draw equals the oracle's on that cache's logits."""
+    cfg_a = gpu.engine.config("tiny", max_pos=64)
+    cfg_b = gpu.engine.config("tiny", max_pos=64, vocab=1024)
+    model_a = gpu.engine.Model.seeded(cfg_a, 31).to_device()
+    model_b = gpu.engine.Model.seeded(cfg_b, 32).to_device()
+    eng_a, eng_b = gpu.engine.Engine(model_a, cfg_a), gpu.engine.Engine(model_b, cfg_b)
+    eng_b.sampler_config(1.1, 20, 0.8)
+    eng_a.set_sampling(True)
+    eng_b.set_sampling(True)
+    libc = C.CDLL("libc.so.6")
+    libc.srand(5)
+    rnd = orc.Rand(5)
+    seq_a = [int(t) for t in gpu.engine.seeded_tokens(1, 7, cfg_a.vocab)]
+    seq_b = [int(t) for t in gpu.engine.seeded_tokens(2, 9, cfg_b.vocab)]
+    for _ in range(6):
+        ta = eng_a.inference(seq_a)
+        assert ta == orc.sample(eng_a.host_logits(), rnd)
+        seq_a.append(ta)
+        tb = eng_b.inference(seq_b)
+        assert 0 <= tb < cfg_b.vocab and tb == orc.sample(eng_b.host_logits(), rnd, 1.1, 20, 0.8)
+        seq_b.append(tb)
+    libc.srand(1)
+    for e in (eng_a, eng_b):
+        e.close()
+    for m in (model_a, model_b):
+        m.close()
+
+
+def test_cache_follows_a_change_of_model(gpu):
+    """A cache whose decode graph was captured with one model is then driven with another model of the
+    same configuration: the graph is captured again, the ids are those of a fresh cache on that model."""
+    cfg = gpu.engine.config("tiny", max_pos=64)
+    m1 = gpu.engine.Model.seeded(cfg, 41).to_device()
+    m2 = gpu.engine.Model.seeded(cfg, 42).to_device()
+    prompt = gpu.engine.seeded_tokens(3, 8, cfg.vocab)
+    eng = gpu.engine.Engine(m1, cfg, use_graph=True)
+    a1, _ = eng.generate(prompt, 6)
+    eng.reset()
+    eng.model = m2
+    a2, _ = eng.generate(prompt, 6)
+    ref = gpu.engine.Engine(m2, cfg, use_graph=False)
+    b2, _ = ref.generate(prompt, 6)
+    assert list(a2) == list(b2) and list(a1) != list(a2)
+    eng.close()
+    ref.close()
+    m1.close()
+    m2.close()
+
+
 def test_decode_across_the_long_context_attention_switch(gpu):
     """Greedy decoding from position 500 to 560 changes attention kernels at 512 cached positions (one
     launch before, span + merge launches after) and graphs with them: same ids with and without graphs,

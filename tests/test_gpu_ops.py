@@ -3,6 +3,8 @@ seeded inputs, through the C-ABI.  Integer/byte work (conversion, gather,
 argmax) is bit-exact; floating-point ops stay inside the 2e-2 max-abs/rel
 tolerance the task states, and tighter bounds are asserted where the kernel
 was built to reproduce the oracle's bits (RMSNorm, RoPE, residual)."""
+import ctypes as C
+
 import numpy as np
 import pytest
 
@@ -180,6 +182,34 @@ def test_linear_gemm_ragged_shapes(gpu, T, K, N):
     assert e <= TIGHT
     got_r = gpu.ops.linear(x, w, residual=res)
     assert H.mixed_err(got_r, orc.add(orc.linear(x, w), res)) <= TOL
+
+
+def test_split_k_linear_on_two_streams_at_once(gpu):
+    """Split-K projections (64 rows, few output tiles) issued on two streams without waiting in between:
+    each stream has its own partial-sum buffer, so both results equal the single-stream result bit for bit."""
+    L, cap = gpu.lib(), gpu.capi
+    T, K, N = 64, 4096, 4096
+    streams = []
+    for _ in range(2):
+        s = C.c_void_p()
+        cap.check(L.llm_stream_create(C.byref(s)))
+        streams.append(s)
+    bufs, want = [], []
+    for i in range(2):
+        x, w = _proj_inputs(50 + i, T, K, N)
+        want.append(gpu.ops.linear(x, w))   # default stream, alone
+        bufs.append((cap.DevBuf.from_host(x), cap.DevBuf.from_host(w), cap.DevBuf((T, N), np.uint16)))
+    for rep in range(20):
+        for i in range(2):
+            d_x, d_w, d_o = bufs[i]
+            cap.check(L.llm_linear(d_x.ptr, K, d_w.ptr, None, 0, d_o.ptr, N, T, N, K, streams[i]))
+    for s in streams:
+        cap.check(L.llm_stream_sync(s))
+    for i in range(2):
+        assert np.array_equal(bufs[i][2].download(), want[i]), i
+        assert H.mixed_err(want[i], orc.linear(*_proj_inputs(50 + i, T, K, N))) <= TIGHT
+    for s in streams:
+        cap.check(L.llm_stream_destroy(s))
 
 
 def test_linear_gemm_reference_test_operand_pattern(gpu):

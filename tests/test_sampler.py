@@ -183,3 +183,68 @@ def test_fast_head_selection_equals_the_full_sort_path(pkg):
         print("vocab %d: head selection %.3f ms per token, full sort %.3f ms" % (vocab, 1e3 * (t1 - t0) / n, 1e3 * (t2 - t1) / n))
     lib.llama3_sampler_config(128256, 0.7, 50, 0.9)
     libc.srand(1)
+
+
+def test_two_vocabularies_interleaved_do_not_share_settings(pkg):
+    """The settings-carrying sampler reads no process-wide state: draws for a 4096-entry and a
+    128256-entry vocabulary alternate on exactly-sized buffers while the process-wide setting names a
+    third size, and each equals the oracle's draw."""
+    lib = pkg.lib()
+    libc = C.CDLL("libc.so.6")
+    rng = np.random.default_rng(8)
+    lib.llama3_sampler_config(777, 0.7, 50, 0.9)
+    libc.srand(3)
+    r = orc.Rand(3)
+    for i in range(8):
+        vocab = (4096, 128256)[i % 2]
+        lg = _logits(rng, vocab, scale=2.0)
+        scratch = np.empty(vocab, np.float32)
+        got = lib.llama3_sample_with(vocab, 0.7, 50, 0.9, scratch.ctypes.data, lg.ctypes.data)
+        assert got == orc.sample(lg, r)
+    lib.llama3_sampler_config(128256, 0.7, 50, 0.9)
+    libc.srand(1)
+
+
+def test_sampler_sources_under_address_sanitizer(tmp_path):
+    """The host sampler compiled with -fsanitize=address (host code only) and driven with two
+    vocabulary sizes alternately on heap buffers of exactly those sizes, through the settings-carrying
+    call and through the reference-named call after llama3_sampler_config: any read or write past a
+    buffer aborts the program."""
+    import os
+    import shutil
+    import subprocess
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    src = os.path.join(root, "llm.cu_amd", "src")
+    main = tmp_path / "main.cpp"
+    main.write_text(r'''
+#include <cstdio>
+#include <cstdlib>
+#include <vector>
+#include "llama3_host.h"
+extern "C" const char *llm_last_error(void) { return ""; }  // the kernel library is not part of this build
+int main() {
+    const int sizes[2] = {4096, 128256};
+    long acc = 0;
+    for (int it = 0; it < 6; ++it) {
+        const int v = sizes[it % 2];
+        std::vector<llm_half> lg(v);
+        std::vector<float> scratch(v);
+        for (int i = 0; i < v; ++i) lg[i] = (llm_half)(0x3000 + (i * 2654435761u >> 20) % 0x0c00); // 0.125 .. 4
+        acc += llama3_sample_with(v, 0.7f, 50, 0.9f, scratch.data(), lg.data());
+        acc += llama3_sample_with(v, 1.3f, 0, 0.5f, scratch.data(), lg.data());   // full-sort path
+        llama3_sampler_config(v, 0.7f, 50, 0.9f);
+        acc += sample_next_token(scratch.data(), lg.data());
+        acc += sample_next_token_reference(scratch.data(), lg.data());
+    }
+    printf("ok %ld\n", acc);
+    return 0;
+}
+''')
+    exe = tmp_path / "sampler_asan"
+    cmd = [shutil.which("g++") or "g++", "-O1", "-g", "-std=c++17", "-fsanitize=address", "-fno-omit-frame-pointer",
+           "-fopenmp", "-I", os.path.join(root, "include"), "-I", src, str(main),
+           os.path.join(src, "inference", "sampler.cpp"), os.path.join(src, "common", "fail.cpp"), "-o", str(exe)]
+    subprocess.check_call(cmd)
+    env = dict(os.environ, ASAN_OPTIONS="detect_leaks=0", LD_PRELOAD="")
+    out = subprocess.run([str(exe)], env=env, capture_output=True, text=True, timeout=120)
+    assert out.returncode == 0 and out.stdout.startswith("ok"), out.stderr[-2000:]
