@@ -177,6 +177,25 @@ int llm_attn_decode_rope(const uint16_t *qkv_dev, uint16_t *k_cache_dev, uint16_
                          uint16_t *out_dev, int pos_host, const int32_t *pos_dev, const float *table_dev,
                          int n_heads, int n_kv_heads, int head_dim, int max_pos, void *workspace_dev,
                          llm_stream_t stream);
+/* llm_attn_decode_rope and the projection that consumes its result (compute_output + add_norm,
+ * src/inference/inference.cu:600-618,366-390) in one launch, for positions below 512: the first
+ * workgroups compute the attention into attn_out_dev ([Hq*hd]) exactly as llm_attn_decode_rope does;
+ * all others fetch their rows of w ([N, Hq*hd]) while the attention runs, wait for its output, and
+ * write out[n] = fp16(fp16(sum_k attn[k] * w[n,k]) + residual[n]) (residual may be NULL or alias out).
+ * Same bits as llm_attn_decode_rope followed by llm_linear with T = 1 (a NaN result of the attention
+ * may differ in its payload bits).
+ * attn_out_dev must hold the "empty" pattern when the launch starts: llm_attn_oproj_buffer_init() once,
+ * after that every launch refills attn_out_next_dev, the buffer that the next such launch in stream
+ * order will pass as attn_out_dev (a ring of two or more buffers; never the same as attn_out_dev).
+ * timeouts_dev: one int32, zeroed by the caller, counts waits that gave up (must stay 0).
+ * Launches that share these buffers must not overlap.  Limits: Hq*hd <= 4096, N <= 24 * (CUs - Hkv*4). */
+int llm_attn_oproj_supported(int n_heads, int n_kv_heads, int head_dim, int N); /* 1 or 0, current device */
+int llm_attn_oproj_buffer_init(uint16_t *buf_dev, int n, llm_stream_t stream);
+int llm_attn_decode_rope_oproj(const uint16_t *qkv_dev, uint16_t *k_cache_dev, uint16_t *v_cache_dev,
+                               uint16_t *attn_out_dev, uint16_t *attn_out_next_dev, int pos_host,
+                               const int32_t *pos_dev, const float *table_dev, int n_heads, int n_kv_heads,
+                               int head_dim, int max_pos, const uint16_t *w_dev, const uint16_t *residual_dev,
+                               uint16_t *out_dev, int N, int32_t *timeouts_dev, llm_stream_t stream);
 /* The same operation as two launches: one workgroup per (KV head, 256-position span) leaves partial
  * softmax statistics and P.V, a second kernel (one workgroup per query head) merges them.  Correct at
  * any position; faster than the single launch beyond 512 cached positions (no in-kernel merge tail). */

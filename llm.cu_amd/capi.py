@@ -117,6 +117,9 @@ HIP_ABI = {
     "llm_norm_linear_swiglu": (_i, [_vp, _vp, C.c_double, _vp, _vp, _vp, _i, _i, _vp]),
     "llm_attn_decode_rope": (_i, [_vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _vp, _vp]),
     "llm_attn_decode_rope_batch": (_i, [_vp, _i, _vp, _vp, _vp, _i, _vp, _i, _vp, _i, _i, _i, _i, _vp, _vp]),
+    "llm_attn_oproj_supported": (_i, [_i, _i, _i, _i]),
+    "llm_attn_oproj_buffer_init": (_i, [_vp, _i, _vp]),
+    "llm_attn_decode_rope_oproj": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _vp, _vp, _vp, _i, _vp, _vp]),
     "llm_attn_decode_rope_long": (_i, [_vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _vp, _vp]),
     "llm_norm_lmhead_argmax": (_i, [_vp, _vp, C.c_double, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp, _vp]),
     "llm_attn_decode_workspace_bytes": (_sz, [_i, _i]),

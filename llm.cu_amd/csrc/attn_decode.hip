@@ -46,11 +46,11 @@ struct AdArgs {
 // that write.
 //
 // NDIM is the number of head dims this workgroup produces, LS the span length.
-template <int HD, int G, bool FUSED, int NDIM, int LS, bool TWOPASS = false>
+template <int HD, int G, bool FUSED, int NDIM, int LS, bool TWOPASS = false, bool AGENT_OUT = false>
 __device__ __forceinline__ void attn_decode_body(const AdArgs &a, float *sc, half_t *qs, half_t *knew, half_t *vnew,
                                                  float *s_m, float *s_l, int *s_last, const int pos,
                                                  const int n_active, const int split, const int d_begin,
-                                                 const bool appender) {
+                                                 const bool appender, const int kvh_arg = -1) {
     constexpr int LPP = HD / 8;                    // lanes per position in the score pass
     constexpr int PPW = 64 / LPP;                  // positions per wavefront pass
     constexpr int KIT = LS / (AD_WAVES * PPW);  // K loads per thread
@@ -62,7 +62,7 @@ __device__ __forceinline__ void attn_decode_body(const AdArgs &a, float *sc, hal
     constexpr int VIT = LS / (JL * 8);          // V loads per thread and pass
     constexpr int HALF = HD / 2;
 
-    const int kvh = blockIdx.x, splits = a.splits;
+    const int kvh = kvh_arg >= 0 ? kvh_arg : (int)blockIdx.x, splits = a.splits;
     const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
     const int max_pos = a.max_pos;
     const int ctx = pos + 1;
@@ -217,11 +217,32 @@ __device__ __forceinline__ void attn_decode_body(const AdArgs &a, float *sc, hal
         if (jc == 0) {
             if (n_active == 1 && !TWOPASS) {
 #pragma unroll
-                for (int h = 0; h < G; ++h) a.out[(size_t)(kvh * G + h) * HD + d] = (half_t)(acc[h] / s_l[h]);
+                for (int h = 0; h < G; ++h) {
+                    const half_t r = (half_t)(acc[h] / s_l[h]);
+                    if (AGENT_OUT) { // collected in LDS (the queries are no longer needed), stored wide below
+                        uint16_t bits = __builtin_bit_cast(uint16_t, r);
+                        if (bits == 0xFFFFu) bits = 0xFFFEu; // 0xFFFF marks "not written yet" for the reader
+                        reinterpret_cast<uint16_t *>(qs)[h * NDIM + (d - d_begin)] = bits;
+                    }
+                    else
+                        a.out[(size_t)(kvh * G + h) * HD + d] = r;
+                }
             } else {
 #pragma unroll
                 for (int h = 0; h < G; ++h) a.ws_acc[(((size_t)kvh * splits + split) * G + h) * HD + d] = acc[h];
             }
+        }
+    }
+    if (AGENT_OUT) {
+        // This workgroup's G x NDIM results go out as 8-byte device-scope stores (written through to the
+        // point where every XCD reads them): 2-byte write-through stores cost a read-modify-write each.
+        static_assert(!AGENT_OUT || NDIM % 4 == 0, "results are stored four at a time");
+        __syncthreads();
+        if (tid < G * NDIM / 4) {
+            const int h = tid / (NDIM / 4), q = tid % (NDIM / 4);
+            const unsigned long long v = reinterpret_cast<const unsigned long long *>(qs)[tid];
+            __hip_atomic_store(reinterpret_cast<unsigned long long *>(a.out + (size_t)(kvh * G + h) * HD + d_begin) + q, v,
+                               __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
     }
     if (n_active == 1 && !TWOPASS) return;
@@ -307,6 +328,162 @@ __global__ __launch_bounds__(AD_THREADS) void attn_decode_kernel(const AdArgs a)
         attn_decode_body<HD, G, FUSED, HD, AD_LS>(a, sc, qs, knew, vnew, s_m, s_l, &s_last, pos, n_active, y, 0,
                                                   y == n_active - 1);
     }
+}
+
+// ---------------------------------------------------------------------------
+// Attention of one token and the projection that consumes it, in one launch.
+//
+// The attention above occupies Hkv * DSN workgroups for a few microseconds and moves about a megabyte:
+// HBM idles meanwhile, and the output projection launched behind it then pays its own launch, its own
+// first trip to HBM and the streaming of its whole matrix.  Here the workgroups with the lowest ids run
+// the attention exactly as above; every other workgroup belongs to the projection: it asks for all of its
+// weight rows at once (they stay in registers), and only then waits for the attention output, stages it
+// in LDS and reduces.  Streaming the matrix thus overlaps the attention.
+//
+// Hand-over without counters or fences: the attention output buffer starts out filled with a 16-bit
+// pattern that the attention never writes (AO_EMPTY, a NaN; a result with those bits is stored with the
+// lowest bit cleared).  The attention stores its results write-through at device scope; the projection
+// workgroups read the buffer with device-scope loads until no word holds the pattern any more: the data
+// is its own flag.  The launch refills `next`, the buffer of the following launch in stream order (the
+// host passes a ring of at least two buffers), so every launch finds its own buffer empty.
+// One workgroup per CU at most (grid <= number of CUs), and workgroups are dispatched in id order, so the
+// attention workgroups are running before any projection workgroup can wait for them: the wait cannot
+// deadlock.  It is bounded anyway (AO_SPIN_LIMIT rounds, after which the workgroup carries on and counts
+// a timeout in *timeouts for the host to see).
+// ---------------------------------------------------------------------------
+#define AO_WAVES 8          // = AD_WAVES: both roles use 512 threads
+#define AO_ROWS 3           // weight rows per wavefront of the projection part, at most
+#define AO_KSTEPS 8         // 16-byte loads per lane and row: K <= 4096
+#define AO_SPIN_LIMIT (1 << 18)
+#define AO_EMPTY 0xFFFFu
+
+struct AoArgs {
+    const half_t *w;   // [N, K] projection weights
+    const half_t *res; // [N] residual (may alias out) or null
+    half_t *out;       // [N]
+    uint16_t *next;    // [K] attention output buffer of the next launch: refilled with AO_EMPTY here
+    int N, K;
+    int n_owg;         // projection workgroups
+    int rows;          // weight rows per wavefront (<= AO_ROWS)
+    int *timeouts;     // diagnostic: waits that ran into AO_SPIN_LIMIT
+};
+
+template <int HD, int G, int DSN>
+__global__ __launch_bounds__(AD_THREADS) void attn_oproj_kernel(const AdArgs a, const AoArgs o) {
+    __shared__ float sc[G * AD_LS];
+    __shared__ __attribute__((aligned(16))) half_t qs[G * HD];
+    __shared__ __attribute__((aligned(16))) half_t knew[HD];
+    __shared__ __attribute__((aligned(16))) half_t vnew[HD];
+    __shared__ float s_m[G], s_l[G];
+    __shared__ int s_last;
+    const int n_attn = a.n_kv_heads * DSN;
+    const int wg = blockIdx.x, tid = threadIdx.x;
+    if (wg < n_attn) {
+        int pos = a.pos_host + (a.pos_dev ? *a.pos_dev : 0);
+        if (pos > a.max_pos - 1) pos = a.max_pos - 1;
+        if (pos > AD_LS - 1) pos = AD_LS - 1; // this form serves one span; the host picks it below AD_LS only
+        if (pos < 0) pos = 0;
+        const int kvh = wg % a.n_kv_heads, y = wg / a.n_kv_heads;
+        attn_decode_body<HD, G, true, HD / DSN, AD_LS, false, true>(a, sc, qs, knew, vnew, s_m, s_l, &s_last, pos, 1, 0,
+                                                                    y * (HD / DSN), y == 0, kvh);
+        // off the critical path: the next launch's buffer back to "empty" (visible at the end of this kernel)
+        uint32_t *nx = reinterpret_cast<uint32_t *>(o.next);
+        for (int c = wg * AD_THREADS + tid; c < o.K / 2; c += n_attn * AD_THREADS) nx[c] = AO_EMPTY | (AO_EMPTY << 16);
+        return;
+    }
+    // ---- projection part ----------------------------------------------------------------
+    half_t *xs = reinterpret_cast<half_t *>(sc); // K halves: K * 2 <= sizeof(sc), checked by the host
+    const int wave = tid / 64, lane = tid % 64;
+    const int K = o.K, N = o.N;
+    const int wslot = (wg - n_attn) * AO_WAVES + wave; // this wavefront among all of the projection part
+    const int wtotal = o.n_owg * AO_WAVES;
+    half8_t wreg[AO_ROWS][AO_KSTEPS];
+    half_t resv[AO_ROWS];
+    // a head start of about a microsecond for the attention's own loads (measured: 12.2 -> 11.4 us per launch)
+    for (int dl = 0; dl < 5; ++dl) __builtin_amdgcn_s_sleep(8);
+#pragma unroll
+    for (int r = 0; r < AO_ROWS; ++r) {
+        int row = wslot + wtotal * r; // adjacent wavefronts read adjacent rows
+        const bool live = r < o.rows && row < N;
+        row = live ? row : N - 1;
+#pragma unroll
+        for (int j = 0; j < AO_KSTEPS; ++j) {
+            const int k = lane * 8 + 512 * j;
+            wreg[r][j] = (live && k < K) ? load8_nt(o.w + (size_t)row * K + k) : half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+        }
+        resv[r] = (live && o.res) ? o.res[row] : (half_t)0.f;
+    }
+    // ---- the attention output, as soon as it is there ------------------------------------
+    {
+        const uint32_t *src = reinterpret_cast<const uint32_t *>(a.out);
+        uint32_t *dst = reinterpret_cast<uint32_t *>(xs);
+        // K/2 words over 512 threads: at most AO_KSTEPS/2 per thread, all asked for in one round
+        constexpr int WPT = AO_KSTEPS * 512 / 2 / AD_THREADS;
+        uint32_t v[WPT];
+        int spins = 0;
+        for (;;) {
+            bool empty = false;
+#pragma unroll
+            for (int i = 0; i < WPT; ++i) {
+                const int c = tid + AD_THREADS * i;
+                v[i] = c < K / 2 ? __hip_atomic_load(src + c, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0u;
+            }
+#pragma unroll
+            for (int i = 0; i < WPT; ++i) empty |= (v[i] & 0xFFFFu) == AO_EMPTY || (v[i] >> 16) == AO_EMPTY;
+            if (!empty) break;
+            if (++spins > AO_SPIN_LIMIT) {
+                atomicAdd(o.timeouts, 1);
+                break;
+            }
+            __builtin_amdgcn_s_sleep(2);
+        }
+#pragma unroll
+        for (int i = 0; i < WPT; ++i) {
+            const int c = tid + AD_THREADS * i;
+            if (c < K / 2) dst[c] = v[i];
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < AO_ROWS; ++r) {
+        const int row = wslot + wtotal * r;
+        float acc = 0.f;
+#pragma unroll
+        for (int j = 0; j < AO_KSTEPS; ++j) {
+            const int k = lane * 8 + 512 * j;
+            if (k < K) acc = dot8(wreg[r][j], load8(xs + k), acc);
+        }
+        acc = wave_sum(acc);
+        if (lane == 0 && r < o.rows && row < N) {
+            half_t h = (half_t)acc;
+            if (o.res) h = (half_t)((float)h + (float)resv[r]); // the reference's add_norm on the stored projection
+            o.out[row] = h;
+        }
+    }
+}
+
+template <int HD, int G>
+static int launch_attn_oproj(AdArgs a, AoArgs o, hipStream_t s) {
+    constexpr int DSN = HD >= 128 ? 4 : 1;
+    static_assert(AO_WAVES == AD_WAVES, "both roles share the workgroup size");
+    LLM_REQUIRE((size_t)o.K * sizeof(half_t) <= sizeof(float) * G * AD_LS, "llm_attn_decode_rope_oproj: K=%d does not fit the staging buffer", o.K);
+    int cus = 0;
+    int rc = llm_cu_count_cached(&cus);
+    if (rc != LLM_OK) return rc;
+    const int n_attn = a.n_kv_heads * DSN;
+    LLM_REQUIRE(cus > n_attn, "llm_attn_decode_rope_oproj: %d attention workgroups on %d CUs", n_attn, cus);
+    // at most one workgroup per CU: all of them are resident at once
+    int owg = (o.N + AO_WAVES - 1) / AO_WAVES;
+    if (owg > cus - n_attn) owg = cus - n_attn;
+    const int rows = (o.N + owg * AO_WAVES - 1) / (owg * AO_WAVES);
+    LLM_REQUIRE(rows <= AO_ROWS, "llm_attn_decode_rope_oproj: N=%d needs %d rows per wavefront on %d CUs (at most %d)", o.N, rows,
+                cus, AO_ROWS);
+    o.n_owg = owg;
+    o.rows = rows;
+    a.splits = 1;
+    attn_oproj_kernel<HD, G, DSN><<<dim3(n_attn + owg), dim3(AD_THREADS), 0, s>>>(a, o);
+    LLM_LAUNCH_CHECK("attn_oproj_kernel");
+    return LLM_OK;
 }
 
 template <int HD, int G, bool FUSED>
@@ -670,6 +847,85 @@ int llm_attn_decode_rope(const uint16_t *qkv, uint16_t *kc, uint16_t *vc, uint16
     a.n_kv_heads = n_kv_heads;
     a.max_pos = max_pos;
     return dispatch_decode<true>(a, n_heads, head_dim, workspace, (hipStream_t)stream);
+}
+
+int llm_attn_decode_rope_oproj(const uint16_t *qkv, uint16_t *kc, uint16_t *vc, uint16_t *attn_out, uint16_t *attn_out_next,
+                               int pos_host, const int32_t *pos_dev, const float *table, int n_heads, int n_kv_heads,
+                               int head_dim, int max_pos, const uint16_t *w, const uint16_t *residual, uint16_t *out, int N,
+                               int32_t *timeouts_dev, llm_stream_t stream) {
+    LLM_REQUIRE(qkv && kc && vc && attn_out && attn_out_next && table && w && out && timeouts_dev,
+                "llm_attn_decode_rope_oproj: null pointer");
+    LLM_REQUIRE(attn_out != attn_out_next, "llm_attn_decode_rope_oproj: a launch cannot refill its own buffer");
+    LLM_REQUIRE(n_kv_heads > 0 && n_heads % n_kv_heads == 0, "llm_attn_decode_rope_oproj: heads %d/%d", n_heads, n_kv_heads);
+    LLM_REQUIRE(max_pos > 0 && max_pos % 64 == 0, "llm_attn_decode_rope_oproj: max_pos=%d must be a multiple of 64", max_pos);
+    LLM_REQUIRE(pos_dev || (pos_host >= 0 && pos_host < max_pos && pos_host < AD_LS),
+                "llm_attn_decode_rope_oproj: position %d (must be below %d and below max_pos %d)", pos_host, AD_LS, max_pos);
+    const int K = n_heads * head_dim;
+    LLM_REQUIRE(N > 0 && K % 8 == 0 && K <= 512 * AO_KSTEPS, "llm_attn_decode_rope_oproj: N=%d K=%d (K <= %d)", N, K,
+                512 * AO_KSTEPS);
+    LLM_REQUIRE(aligned16(qkv) && aligned16(kc) && aligned16(vc) && aligned16(attn_out) && aligned16(attn_out_next) &&
+                    aligned16(w),
+                "llm_attn_decode_rope_oproj: pointers must be 16-byte aligned");
+    AdArgs a = {};
+    a.q = (const half_t *)qkv;
+    a.kc = (half_t *)kc;
+    a.vc = (half_t *)vc;
+    a.out = (half_t *)attn_out;
+    a.table = table;
+    a.pos_host = pos_host;
+    a.pos_dev = pos_dev;
+    a.n_kv_heads = n_kv_heads;
+    a.max_pos = max_pos;
+    AoArgs o = {};
+    o.w = (const half_t *)w;
+    o.res = (const half_t *)residual;
+    o.out = (half_t *)out;
+    o.next = attn_out_next;
+    o.N = N;
+    o.K = K;
+    o.timeouts = timeouts_dev;
+    hipStream_t s = (hipStream_t)stream;
+    const int G = n_heads / n_kv_heads;
+#define AO_CASE(HD_, G_) \
+    if (head_dim == HD_ && G == G_) return launch_attn_oproj<HD_, G_>(a, o, s);
+    AO_CASE(128, 4)
+    AO_CASE(128, 8)
+    AO_CASE(128, 1)
+    AO_CASE(64, 4)
+    AO_CASE(64, 1)
+    AO_CASE(32, 4)
+    AO_CASE(32, 1)
+#undef AO_CASE
+    llm_set_error("llm_attn_decode_rope_oproj: head_dim=%d with group size %d is not built", head_dim, G);
+    return LLM_ERR_INVALID;
+}
+
+// 1 when llm_attn_decode_rope_oproj covers these shapes on the current device, else 0.
+int llm_attn_oproj_supported(int n_heads, int n_kv_heads, int head_dim, int N) {
+    if (n_kv_heads <= 0 || n_heads % n_kv_heads) return 0;
+    const int G = n_heads / n_kv_heads, K = n_heads * head_dim;
+    if (!((head_dim == 128 && (G == 1 || G == 4 || G == 8)) || ((head_dim == 64 || head_dim == 32) && (G == 1 || G == 4)))) return 0;
+    if (K % 8 || K > 512 * AO_KSTEPS || (size_t)K * sizeof(half_t) > sizeof(float) * G * AD_LS || N <= 0) return 0;
+    int cus = 0;
+    if (llm_cu_count_cached(&cus) != LLM_OK) return 0;
+    const int n_attn = n_kv_heads * (head_dim >= 128 ? 4 : 1);
+    if (cus <= n_attn) return 0;
+    int owg = (N + AO_WAVES - 1) / AO_WAVES;
+    if (owg > cus - n_attn) owg = cus - n_attn;
+    return (N + owg * AO_WAVES - 1) / (owg * AO_WAVES) <= AO_ROWS;
+}
+
+// Fills n fp16 slots with the "not written yet" pattern of llm_attn_decode_rope_oproj (a fill kernel:
+// safe under graph capture).
+__global__ void ao_fill_empty_kernel(uint16_t *p, int n) {
+    int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = AO_EMPTY;
+}
+int llm_attn_oproj_buffer_init(uint16_t *buf, int n, llm_stream_t stream) {
+    LLM_REQUIRE(buf && n > 0, "llm_attn_oproj_buffer_init: buf/n");
+    ao_fill_empty_kernel<<<dim3((n + 255) / 256), dim3(256), 0, (hipStream_t)stream>>>(buf, n);
+    LLM_LAUNCH_CHECK("ao_fill_empty_kernel");
+    return LLM_OK;
 }
 
 int llm_attn_decode_rope_long(const uint16_t *qkv, uint16_t *kc, uint16_t *vc, uint16_t *out, int pos_host,

@@ -102,6 +102,16 @@ __global__ __launch_bounds__(GEMV_THREADS) void gemv_kernel(const GemvArgs a) {
     }
     issue_next(0);
     issue_next(1);
+    // the residual of each of this wavefront's rows, asked for now: at the end of a row the value is
+    // there instead of one more trip to memory behind the last weight load
+    half_t resv[4] = {(half_t)0.f, (half_t)0.f, (half_t)0.f, (half_t)0.f};
+    if (MODE == GV_PLAIN && a.res) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int row = row_base + row_step * r;
+            if (r < a.rpw && row < N) resv[r] = a.res[row];
+        }
+    }
     if (a.gain) {
         rms_finish<GEMV_THREADS, GEMV_NORM_R>(xr, xs, K, a.eps, red);
     } else {
@@ -142,7 +152,14 @@ __global__ __launch_bounds__(GEMV_THREADS) void gemv_kernel(const GemvArgs a) {
                     const unsigned long long c = pack_candidate(h, row);
                     mine = c > mine ? c : mine;
                 } else {
-                    if (lane == 0) a.out[row] = finish(s0, a.res ? a.res + row : nullptr);
+                    if (lane == 0) {
+                        half_t hres = (half_t)s0;
+                        if (a.res) { // fp16(fp16(sum) + residual), the reference's add_norm on the stored projection
+                            const half_t rv = i < 4 ? resv[i < 4 ? i : 0] : a.res[row];
+                            hres = (half_t)((float)hres + (float)rv);
+                        }
+                        a.out[row] = hres;
+                    }
                 }
             }
 #pragma unroll

@@ -247,3 +247,30 @@ def attn_decode_rope(qkv, kc, vc, pos, n_heads, n_kv_heads, head_dim, theta=5000
         check(fn(d_q.ptr, d_k.ptr, d_v.ptr, d_o.ptr, pos, None, d_t.ptr, n_heads, n_kv_heads,
                  head_dim, max_pos, d_ws.ptr, None))
     return d_o.download(), d_k.download(), d_v.download()
+
+
+def attn_decode_rope_oproj(qkv, kc, vc, pos, n_heads, n_kv_heads, head_dim, w, residual=None, theta=500000.0, repeats=1):
+    """llm_attn_decode_rope_oproj: returns (attention output [Hq*hd], projection output [N], K cache, V cache,
+    timeouts).  Each repeat starts from the same caches and uses the next buffer of a two-buffer ring."""
+    qkv, kc, vc, w = _u16(qkv).reshape(-1), _u16(kc), _u16(vc), _u16(w)
+    max_pos = kc.shape[1]
+    N = w.shape[0]
+    qd = n_heads * head_dim
+    d_q, d_t = DevBuf.from_host(qkv), DevBuf.from_host(rope_table(max_pos, head_dim, theta))
+    d_w = DevBuf.from_host(w)
+    ring = DevBuf((2, qd), np.uint16)
+    check(lib().llm_attn_oproj_buffer_init(ring.ptr, 2 * qd, None))
+    tmo = DevBuf((1,), np.int32)
+    tmo.zero()
+    res = None
+    for r in range(repeats):
+        d_k, d_v = DevBuf.from_host(kc), DevBuf.from_host(vc)
+        d_o = DevBuf.from_host(_u16(residual).reshape(-1)) if residual is not None else DevBuf((N,), np.uint16)
+        cur, nxt = ring.ptr + 2 * qd * (r % 2), ring.ptr + 2 * qd * ((r + 1) % 2)
+        check(lib().llm_attn_decode_rope_oproj(d_q.ptr, d_k.ptr, d_v.ptr, cur, nxt, pos, None, d_t.ptr, n_heads, n_kv_heads,
+                                               head_dim, max_pos, d_w.ptr, d_o.ptr if residual is not None else None,
+                                               d_o.ptr, N, tmo.ptr, None))
+        out = (ring.download()[r % 2].copy(), d_o.download(), d_k.download(), d_v.download())
+        assert res is None or all(np.array_equal(x, y) for x, y in zip(res, out)), "repeat %d differs" % r
+        res = out
+    return res + (int(tmo.download()[0]),)

@@ -50,7 +50,8 @@ struct Engine {
     float *rope_table = nullptr;
     int32_t *d_tokens = nullptr; // [max_pos + 1]
     int32_t *d_pos = nullptr;    // tokens cached so far; d_tokens[*d_pos] is the next input
-    int32_t *d_token = nullptr;  // last argmax
+    int32_t *d_token = nullptr;  // [0] last argmax, [1] waits of the fused attention + projection launch that gave up
+    llm_half *ao_ring = nullptr; // one attention-output buffer per layer for llm_attn_decode_rope_oproj (null: not used)
     void *ws_attn = nullptr, *ws_lm = nullptr;
     llm_half *trace_dev = nullptr;
     size_t trace_rows = 0;
@@ -175,10 +176,20 @@ void issue_pass(Engine *e, const Llama3 *m, int T, int pos0, bool dev_pos, bool 
                 llama3_check(llm_norm_linear(e->x, w.in_ln, c.rms_eps, w.wv, e->qkv + qd + kvd, kvd, d, s),
                              "llm_norm_linear(v)");
             }
-            llama3_check((e->long_attn ? llm_attn_decode_rope_long : llm_attn_decode_rope)(
-                             e->qkv, kc, vc, e->attn, p0, pd, e->rope_table, Hq, Hkv, hd, c.max_pos, e->ws_attn, s),
-                         "llm_attn_decode_rope");
-            llama3_check(llm_linear(e->attn, qd, w.wo, e->x, d, e->x, d, 1, d, qd, s), "llm_linear(o)");
+            if (!e->long_attn && e->ao_ring) {
+                // attention and output projection in one launch: the projection's weights stream while the
+                // attention runs.  Layer l hands over through ring buffer l and re-arms the next one.
+                llama3_check(llm_attn_decode_rope_oproj(e->qkv, kc, vc, e->ao_ring + (size_t)l * qd,
+                                                        e->ao_ring + (size_t)((l + 1) % c.n_layers) * qd, p0, pd,
+                                                        e->rope_table, Hq, Hkv, hd, c.max_pos, w.wo, e->x, e->x, d,
+                                                        e->d_token + 1, s),
+                             "llm_attn_decode_rope_oproj");
+            } else {
+                llama3_check((e->long_attn ? llm_attn_decode_rope_long : llm_attn_decode_rope)(
+                                 e->qkv, kc, vc, e->attn, p0, pd, e->rope_table, Hq, Hkv, hd, c.max_pos, e->ws_attn, s),
+                             "llm_attn_decode_rope");
+                llama3_check(llm_linear(e->attn, qd, w.wo, e->x, d, e->x, d, 1, d, qd, s), "llm_linear(o)");
+            }
             llama3_check(llm_norm_linear_swiglu(e->x, w.post_ln, c.rms_eps, w.wg, w.wu, e->ffn, F, d, s),
                          "llm_norm_linear_swiglu");
             llama3_check(llm_linear(e->ffn, F, w.wd, e->x, d, e->x, d, 1, d, F, s), "llm_linear(down)");
@@ -221,6 +232,12 @@ void issue_pass(Engine *e, const Llama3 *m, int T, int pos0, bool dev_pos, bool 
                  "llm_norm_lmhead_argmax");
 }
 
+// h_stage[3] mirrors d_token[1]: waits inside llm_attn_decode_rope_oproj that ran into their limit.  Any
+// such wait means a projection used an incomplete attention output: fail loudly.
+void check_handover(Engine *e) {
+    if (e->h_stage[3] != 0) llama3_fail("attention/projection hand-over timed out %d time(s)", e->h_stage[3]);
+}
+
 // Appends n host tokens at e->pos with one multi-row pass.  Leaves
 // d_pos = pos + n and d_tokens[pos + n] = the greedy next token.
 // logits_host (may be null): pinned host memory that receives the fp16 logits before the pass's one sync.
@@ -257,13 +274,14 @@ int run_pass(Engine *e, const Llama3 *m, const int *tokens, int n, llm_half *log
     }
     e->long_attn = n == 1 && e->pos >= LONG_ATTN_FROM; // single rows go through the decode kernels
     issue_pass(e, m, n, e->pos, false, trace, inject);
-    llama3_check(llm_memcpy_d2h(&e->h_stage[2], e->d_token, sizeof(int32_t), s), "D2H token");
+    llama3_check(llm_memcpy_d2h(&e->h_stage[2], e->d_token, sizeof(int32_t) * 2, s), "D2H token");
     if (trace)
         llama3_check(llm_memcpy_d2h(e->trace_host, e->trace_dev, sizeof(llm_half) * (size_t)c.n_layers * n * c.d_model, s),
                      "D2H trace");
     if (logits_host)
         llama3_check(llm_memcpy_d2h(logits_host, e->logits, sizeof(llm_half) * (size_t)c.vocab, s), "D2H logits");
     llama3_check(llm_stream_sync(s), "stream sync");
+    check_handover(e);
     e->trace_host = nullptr;
     e->inject_host = nullptr;
     e->tokens.insert(e->tokens.end(), tokens, tokens + n);
@@ -316,10 +334,11 @@ int step_one(Engine *e, const Llama3 *m, int token, llm_half *logits_host) {
         llama3_check(llm_memcpy_h2d(e->d_pos, &e->h_stage[1], sizeof(int32_t), s), "H2D position");
     }
     launch_decode_step(e, m, e->pos);
-    llama3_check(llm_memcpy_d2h(&e->h_stage[2], e->d_token, sizeof(int32_t), s), "D2H token");
+    llama3_check(llm_memcpy_d2h(&e->h_stage[2], e->d_token, sizeof(int32_t) * 2, s), "D2H token");
     if (logits_host)
         llama3_check(llm_memcpy_d2h(logits_host, e->logits, sizeof(llm_half) * (size_t)c.vocab, s), "D2H logits");
     llama3_check(llm_stream_sync(s), "stream sync");
+    check_handover(e);
     e->tokens.push_back(token);
     e->pos += 1;
     e->dev_pos_valid = true;
@@ -364,7 +383,12 @@ extern "C" CudaCache *init_cache_cfg(Llama3 *m, const ModelConfig *cfg) {
     }
     e->d_tokens = dmalloc<int32_t>(R + 1, "llm_malloc(tokens)");
     e->d_pos = dmalloc<int32_t>(1, "llm_malloc(pos)");
-    e->d_token = dmalloc<int32_t>(1, "llm_malloc(token)");
+    e->d_token = dmalloc<int32_t>(2, "llm_malloc(token)");
+    llama3_check(llm_fill_zero(e->d_token, sizeof(int32_t) * 2, e->stream), "zero token");
+    if (c.n_layers >= 2 && llm_attn_oproj_supported(c.n_heads, c.n_kv_heads, c.head_dim, d)) {
+        e->ao_ring = dmalloc<llm_half>((size_t)c.n_layers * qd, "llm_malloc(attention hand-over ring)");
+        llama3_check(llm_attn_oproj_buffer_init(e->ao_ring, c.n_layers * qd, e->stream), "llm_attn_oproj_buffer_init");
+    }
     llama3_check(llm_fill_zero(e->d_tokens, sizeof(int32_t) * (R + 1), e->stream), "zero tokens");
     llama3_check(llm_fill_zero(e->d_pos, sizeof(int32_t), e->stream), "zero pos");
     size_t wa = llm_attn_decode_workspace_bytes(c.n_heads, c.head_dim);
@@ -417,7 +441,7 @@ extern "C" void free_cache(CudaCache *C) {
         llm_stream_sync(e->stream);
         drop_graph(e);
         void *bufs[] = {e->x, e->xn, e->qkv, e->attn, e->ffn, e->logits, e->kc, e->vc, e->rope_table,
-                        e->d_tokens, e->d_pos, e->d_token, e->ws_attn, e->ws_lm, e->trace_dev, e->inject_dev,
+                        e->d_tokens, e->d_pos, e->d_token, e->ao_ring, e->ws_attn, e->ws_lm, e->trace_dev, e->inject_dev,
                         e->b_logits, e->b_ids, e->b_ws_attn, e->b_ws_argmax};
         for (void *b : bufs) llm_free(b);
         for (auto ev : e->ev) llm_event_destroy(ev);
@@ -492,7 +516,9 @@ extern "C" int llama3_generate(Llama3 *m, CudaCache *C, const int *prompt, int n
         llama3_check(llm_memcpy_d2h(out_tokens + 1, e->d_tokens + start + n_prompt + 1,
                                     sizeof(int32_t) * (size_t)(n_decode - 1), s),
                      "D2H tokens");
+        llama3_check(llm_memcpy_d2h(&e->h_stage[2], e->d_token, sizeof(int32_t) * 2, s), "D2H token");
         llama3_check(llm_stream_sync(s), "stream sync");
+        check_handover(e);
     }
     // host mirror: the decode steps consumed out_tokens[0..n_decode-2]
     for (int i = 0; i + 1 < n_decode; ++i) e->tokens.push_back(out_tokens[i]);
