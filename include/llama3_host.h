@@ -156,6 +156,14 @@ int llama3_sample_with(int vocab, float temperature, int top_k, float top_p, flo
 /* inference() returns the greedy id (0, default) or sample_next_token() of the logits as the
  * reference does (1). */
 void llama3_set_sampling(CudaCache *c, int on);
+/* 1: decode steps below 512 cached positions run as one launch per token (llm_decode_fused) when the
+ * model shapes and the device allow it; 0 (default): one launch per operation.  Same results bit for
+ * bit; on MI355X the per-operation launches are the faster of the two (305 against 361 tok/s at 8B). */
+void llama3_set_fused_decode(CudaCache *c, int on);
+int llama3_fused_decode_active(const CudaCache *c);
+/* The vectors the last one-launch token passed between its phases, all layers: which = 0 qkv, 1 attention
+ * output, 2 x after O, 3 FFN hidden vector, 4 layer output; out: [n_layers][width] fp16. */
+void llama3_read_fused_vectors(CudaCache *c, int which, llm_half *out);
 
 typedef struct {
     int n_layers;

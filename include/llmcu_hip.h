@@ -219,6 +219,49 @@ int llm_attn_prefill(const uint16_t *q_dev, int ldq, const uint16_t *k_cache_dev
                      const uint16_t *v_cache_dev, uint16_t *out_dev, int ldo, int T, int pos0,
                      int n_heads, int n_kv_heads, int head_dim, int max_pos, llm_stream_t stream);
 
+/* ---- one decode token in one launch ------------------------------------------------------------- */
+/* Replaces, for positions below 512, the whole chain that inference() issues for one new token
+ * (src/inference/inference.cu:149-193 at T = 1: embedding, 32 x {norm, QKV, RoPE, attention, O, +res,
+ * norm, gate/up, down, +res}, final norm, LM head) except the final argmax reduction: one resident
+ * workgroup per CU walks through all phases, the vectors between phases are handed over inside the
+ * kernel.  Logits equal the per-kernel path (llm_norm_linear, llm_attn_decode_rope, llm_linear,
+ * llm_norm_linear_swiglu, llm_norm_lmhead_argmax) bit for bit.
+ * layers_dev: device array of n_layers llm_decode_layer (wqkv = the q, k, v matrices adjacent in memory).
+ * ring_cur_dev / ring_next_dev: two hand-over buffer sets of llm_decode_fused_ring_halves() fp16 each,
+ * both initialised once with llm_attn_oproj_buffer_init(); consecutive tokens alternate them (a launch
+ * works in ring_cur and re-arms ring_next).  The token read is tokens_dev[*pos_dev]; K and V of the
+ * token are appended to the caches at *pos_dev.  phase_begin/phase_end: 0 and llm_decode_fused_phases()
+ * for the whole token (sub-ranges of phases 4*layer + {0 QKV, 1 attention + O, 2 gate/up, 3 down},
+ * last = LM head, are for tests; they use the same ring_cur).  The LM-head phase leaves
+ * llm_decode_fused_candidates() packed argmax candidates in candidates_dev: finish with
+ * llm_argmax_finish().  timeouts_dev: one int32, zeroed by the caller, counts bounded waits that gave up
+ * (must stay 0).  Launches that share buffers must not overlap; nothing else may occupy the GPU's CUs
+ * for long while a launch runs (its workgroups wait for one another). */
+typedef struct {
+    const uint16_t *in_ln, *wqkv, *wo, *post_ln, *wgate, *wup, *wdown;
+    uint16_t *k_cache, *v_cache;
+} llm_decode_layer;
+typedef struct {
+    int n_layers, d_model, n_heads, n_kv_heads, head_dim, ffn_dim, vocab, max_pos;
+    double rms_eps;
+    const float *rope_table_dev;
+    const int32_t *pos_dev, *tokens_dev;
+    const uint16_t *embed_dev, *final_gain_dev, *lm_head_dev;
+    uint16_t *logits_dev;
+    void *candidates_dev;
+} llm_decode_desc;
+int llm_decode_fused_supported(const llm_decode_desc *desc); /* 1 or 0 on the current device */
+size_t llm_decode_fused_ring_halves(const llm_decode_desc *desc);
+int llm_decode_fused_candidates(const llm_decode_desc *desc);
+int llm_decode_fused_phases(const llm_decode_desc *desc);
+int llm_decode_fused(const llm_decode_desc *desc, const llm_decode_layer *layers_dev, uint16_t *ring_cur_dev,
+                     uint16_t *ring_next_dev, int phase_begin, int phase_end, int32_t *timeouts_dev,
+                     llm_stream_t stream);
+/* Final reduction over n packed candidates (as llm_norm_lmhead_argmax does after its GEMV): token_dev,
+ * and tokens_dev[*pos_dev + 1] with *pos_dev incremented when tokens_dev/pos_dev are given. */
+int llm_argmax_finish(const void *candidates_dev, int n, int32_t *token_dev, int32_t *tokens_dev,
+                      int32_t *pos_dev, llm_stream_t stream);
+
 /* ---- LM head + argmax ------------------------------------------------------------ */
 /* Replaces compute_lm_head (src/inference/inference.cu:1003-1028) with the
  * north-star's greedy selection instead of the host sampler: logits =

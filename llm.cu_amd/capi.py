@@ -70,6 +70,17 @@ class CudaCache(C.Structure):
     ]
 
 
+class DecodeLayer(C.Structure):
+    _fields_ = [(k, C.c_void_p) for k in ("in_ln", "wqkv", "wo", "post_ln", "wgate", "wup", "wdown", "k_cache", "v_cache")]
+
+
+class DecodeDesc(C.Structure):
+    _fields_ = [(k, C.c_int) for k in ("n_layers", "d_model", "n_heads", "n_kv_heads", "head_dim", "ffn_dim", "vocab",
+                                       "max_pos")] + [("rms_eps", C.c_double)] + \
+        [(k, C.c_void_p) for k in ("rope_table_dev", "pos_dev", "tokens_dev", "embed_dev", "final_gain_dev", "lm_head_dev",
+                                   "logits_dev", "candidates_dev")]
+
+
 class GenStats(C.Structure):
     _fields_ = [("prefill_ms", C.c_double), ("decode_ms", C.c_double), ("n_prompt", C.c_int),
                 ("n_decode_steps", C.c_int)]
@@ -127,6 +138,12 @@ HIP_ABI = {
     "llm_attn_decode_noalloc_max_bytes": (_sz, []),
     "llm_attn_decode_noalloc": (_i, [_vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _i, _vp]),
     "llm_attn_prefill": (_i, [_vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp]),
+    "llm_decode_fused_supported": (_i, [C.POINTER(DecodeDesc)]),
+    "llm_decode_fused_ring_halves": (_sz, [C.POINTER(DecodeDesc)]),
+    "llm_decode_fused_candidates": (_i, [C.POINTER(DecodeDesc)]),
+    "llm_decode_fused_phases": (_i, [C.POINTER(DecodeDesc)]),
+    "llm_decode_fused": (_i, [C.POINTER(DecodeDesc), _vp, _vp, _vp, _i, _i, _vp, _vp]),
+    "llm_argmax_finish": (_i, [_vp, _i, _vp, _vp, _vp, _vp]),
     "llm_lmhead_workspace_bytes": (_sz, [_i]),
     "llm_lmhead_argmax": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp, _vp]),
     "llm_argmax_f16": (_i, [_vp, _i, _vp, _vp, _vp]),
@@ -185,6 +202,9 @@ HOST_ABI = {
     "top_p_sampling": (_i, [_vp, C.c_float]),
     "llama3_sampler_config": (None, [_i, C.c_float, _i, C.c_float]),
     "llama3_set_sampling": (None, [_CP, _i]),
+    "llama3_set_fused_decode": (None, [_CP, _i]),
+    "llama3_fused_decode_active": (_i, [_CP]),
+    "llama3_read_fused_vectors": (None, [_CP, _i, _vp]),
     "llama3_cache_sampler_config": (None, [_CP, C.c_float, _i, C.c_float]),
     "llama3_sample_with": (_i, [_i, C.c_float, _i, C.c_float, _vp, _vp]),
 }

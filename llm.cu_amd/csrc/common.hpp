@@ -149,3 +149,24 @@ __device__ __forceinline__ uint32_t f16_order_key(uint16_t bits) {
     if (bits == 0x8000u) bits = 0;
     return (bits & 0x8000u) ? (uint32_t)(0x7fffu - (bits & 0x7fffu)) : (uint32_t)(0x8000u + bits);
 }
+
+__device__ __forceinline__ float silu_f(float g) { return g / (1.0f + expf(-g)); }
+
+// fp16(SiLU(gate) * up) as the reference rounds it (src/inference/inference.cu:513-516: the product is an
+// fp32 value, then __float2half): the empty asm keeps the compiler from folding the multiply and the
+// conversion into one instruction that rounds the exact product once (v_fma_mixlo_f16), which differs
+// from the reference's two roundings in the last bit now and then.
+__device__ __forceinline__ half_t swiglu_to_half(float gate, float up) {
+    float p = silu_f(gate) * up;
+    asm volatile("" : "+v"(p));
+    return (half_t)p;
+}
+
+// Candidates are packed (order key + 1) << 32 | ~index so that an unsigned max
+// picks the largest logit and, among equals, the lowest index; NaN packs to 0
+// and never wins.
+__device__ __forceinline__ unsigned long long pack_candidate(half_t h, int idx) {
+    uint16_t bits = __builtin_bit_cast(uint16_t, h);
+    if ((bits & 0x7fffu) > 0x7c00u) return 0ull;
+    return ((unsigned long long)(f16_order_key(bits) + 1u) << 32) | (unsigned long long)(0xffffffffu - (uint32_t)idx);
+}

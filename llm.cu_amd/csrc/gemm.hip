@@ -25,7 +25,6 @@ int gemv_launch(const half_t *x, const half_t *gain, double eps, const half_t *w
 int gemv_swiglu_launch(const half_t *x, const half_t *gain, double eps, const half_t *wg, const half_t *wu,
                        half_t *out, int N, int K, hipStream_t s);
 
-__device__ __forceinline__ float silu_g(float g) { return g / (1.0f + expf(-g)); }
 
 // address-space cast for the LDS side of the loads that go from global memory straight into LDS
 #define DMA_LP(p) ((__attribute__((address_space(3))) void *)(p))
@@ -107,7 +106,7 @@ __global__ __launch_bounds__(SK_WAVES * 64) void skinny_kernel(const half_t *__r
             }
             if (m < T && n < N) {
                 if (SWIGLU) {
-                    out[(size_t)m * ldo + n] = (half_t)(silu_g(s) * s2);
+                    out[(size_t)m * ldo + n] = swiglu_to_half(s, s2);
                 } else {
                     out[(size_t)m * ldo + n] = finish(s, res ? res + (size_t)m * ldr + n : nullptr);
                 }
@@ -257,7 +256,7 @@ __global__ __launch_bounds__(WAVES * 64, 1) void skinny_dma_kernel(const half_t 
                     if (SWIGLU) s2 += red[flip][NW - 1][wv][lane][i];
                 }
                 if (m < T) {
-                    if (SWIGLU) out[(size_t)m * ldo + n] = (half_t)(silu_g(s) * s2);
+                    if (SWIGLU) out[(size_t)m * ldo + n] = swiglu_to_half(s, s2);
                     else out[(size_t)m * ldo + n] = finish(s, res ? res + (size_t)m * ldr + n : nullptr);
                 }
             }
@@ -493,7 +492,7 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_kernel(const half_t *__res
                 const int m = m0 + wm * TM + i * 32 + 8 * (e / 4) + crow0 + (e % 4);
                 if (m < T && n < N) {
                     if (NB == 2) {
-                        out[(size_t)m * ldo + n] = (half_t)(silu_g(acc[0][i][j][e]) * acc[NB - 1][i][j][e]);
+                        out[(size_t)m * ldo + n] = swiglu_to_half(acc[0][i][j][e], acc[NB - 1][i][j][e]);
                     } else {
                         out[(size_t)m * ldo + n] = finish(acc[0][i][j][e], res ? res + (size_t)m * ldr + n : nullptr);
                     }
@@ -783,7 +782,7 @@ __global__ __launch_bounds__(WGM * WGN * 64, OCC) void gemm_dma_kernel(const hal
                 half4_t o;
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
-                    if (NB == 2) o[e] = (half_t)(silu_g(acc[j][i][4 * g + e]) * acc[2 + j][i][4 * g + e]);
+                    if (NB == 2) o[e] = swiglu_to_half(acc[j][i][4 * g + e], acc[2 + j][i][4 * g + e]);
                     else if (res) o[e] = (half_t)((float)(half_t)acc[j][i][4 * g + e] + (float)rv[g][e]);
                     else o[e] = (half_t)acc[j][i][4 * g + e];
                 }
@@ -816,7 +815,7 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float *__restr
     if (NB == 1 && res) r = *reinterpret_cast<const half4_t *>(res + (size_t)m * ldr + n);
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-        if (NB == 2) o[e] = (half_t)(silu_g(a[0][e]) * a[NB - 1][e]);
+        if (NB == 2) o[e] = swiglu_to_half(a[0][e], a[NB - 1][e]);
         else o[e] = res ? (half_t)((float)(half_t)a[0][e] + (float)r[e]) : (half_t)a[0][e];
     }
     *reinterpret_cast<half4_t *>(out + (size_t)m * ldo + n) = o;

@@ -36,17 +36,6 @@ struct GemvArgs {
     int N, K, rpw;
 };
 
-__device__ __forceinline__ float silu_f(float g) { return g / (1.0f + expf(-g)); }
-
-// Candidates are packed (order key + 1) << 32 | ~index so that an unsigned max
-// picks the largest logit and, among equals, the lowest index; NaN packs to 0
-// and never wins.
-__device__ __forceinline__ unsigned long long pack_candidate(half_t h, int idx) {
-    uint16_t bits = __builtin_bit_cast(uint16_t, h);
-    if ((bits & 0x7fffu) > 0x7c00u) return 0ull;
-    return ((unsigned long long)(f16_order_key(bits) + 1u) << 32) | (unsigned long long)(0xffffffffu - (uint32_t)idx);
-}
-
 template <int MODE>
 __global__ __launch_bounds__(GEMV_THREADS) void gemv_kernel(const GemvArgs a) {
     constexpr int NW = MODE == GV_SWIGLU ? 2 : 1; // weight streams per row
@@ -145,7 +134,7 @@ __global__ __launch_bounds__(GEMV_THREADS) void gemv_kernel(const GemvArgs a) {
             float s1 = NW == 2 ? wave_sum(acc[NW - 1]) : 0.f;
             if (row < N) {
                 if (MODE == GV_SWIGLU) {
-                    if (lane == 0) a.out[row] = (half_t)(silu_f(s0) * s1);
+                    if (lane == 0) a.out[row] = swiglu_to_half(s0, s1);
                 } else if (MODE == GV_LMHEAD) {
                     const half_t h = (half_t)s0;
                     if (lane == 0) a.out[row] = h;
@@ -295,6 +284,15 @@ int llm_norm_lmhead_argmax(const uint16_t *x, const uint16_t *gain, double eps, 
     if (rc != LLM_OK) return rc;
     argmax_final_kernel<<<dim3(1), dim3(1024), 0, s>>>((const unsigned long long *)workspace, gemv_blocks(vocab, rpw),
                                                        token, tokens, pos);
+    LLM_LAUNCH_CHECK("argmax_final_kernel");
+    return LLM_OK;
+}
+
+int llm_argmax_finish(const void *candidates, int n, int32_t *token, int32_t *tokens, int32_t *pos, llm_stream_t stream) {
+    LLM_REQUIRE(candidates && token && n > 0, "llm_argmax_finish: candidates/token/n");
+    LLM_REQUIRE((tokens == nullptr) == (pos == nullptr), "llm_argmax_finish: tokens and pos go together");
+    argmax_final_kernel<<<dim3(1), dim3(1024), 0, (hipStream_t)stream>>>((const unsigned long long *)candidates, n, token,
+                                                                         tokens, pos);
     LLM_LAUNCH_CHECK("argmax_final_kernel");
     return LLM_OK;
 }

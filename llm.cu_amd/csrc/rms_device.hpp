@@ -51,8 +51,7 @@ __device__ __forceinline__ void rms_load(const half_t *__restrict__ xrow, const 
 
 // Sum of squares of the loaded row in the reference's order; every thread gets it.
 template <int THREADS, int MAXR>
-__device__ __forceinline__ float rms_sum_squares(const RmsRow<MAXR> &r, int d, float *red) {
-    const int t = threadIdx.x;
+__device__ __forceinline__ float rms_sum_squares(const RmsRow<MAXR> &r, int d, float *red, const int t = threadIdx.x) {
     const int n = d / 4;
     const int R = n >= THREADS ? n / THREADS : 1;
     float p[MAXR];
@@ -107,11 +106,12 @@ __device__ __forceinline__ float rms_from_ss(float ss, int d, double eps) {
 
 // y = fp16((x * g) / rms): multiply, then a correctly rounded divide
 // (inference.cu:355-358).  dst may be global or LDS memory.
+// t: index of the calling thread among the THREADS that share the row (the workgroup's threads by default).
 template <int THREADS, int MAXR>
-__device__ __forceinline__ void rms_finish(const RmsRow<MAXR> &r, half_t *dst, int d, double eps, float *red) {
-    const float ss = rms_sum_squares<THREADS, MAXR>(r, d, red);
+__device__ __forceinline__ void rms_finish(const RmsRow<MAXR> &r, half_t *dst, int d, double eps, float *red,
+                                           const int t = threadIdx.x) {
+    const float ss = rms_sum_squares<THREADS, MAXR>(r, d, red, t);
     const float rms = rms_from_ss(ss, d, eps);
-    const int t = threadIdx.x;
 #pragma unroll
     for (int j = 0; j < MAXR; ++j) {
         if (j < r.R) {

@@ -189,6 +189,23 @@ class Engine:
         lib().llama3_read_batch_logits(self.cache, b, out.ctypes.data)
         return out
 
+    def set_fused_decode(self, on):
+        """One launch per token (True, default where supported) or one launch per operation (False)."""
+        lib().llama3_set_fused_decode(self.cache, 1 if on else 0)
+
+    @property
+    def fused_decode_active(self):
+        return bool(lib().llama3_fused_decode_active(self.cache))
+
+    def fused_vectors(self, which):
+        """Hand-over vectors of the last one-launch token: 0 qkv, 1 attention, 2 x after O, 3 FFN hidden, 4 layer output."""
+        c = self.cfg
+        qd = c.n_heads * c.head_dim
+        width = [qd + 2 * c.n_kv_heads * c.head_dim, qd, c.d_model, c.ffn_dim, c.d_model][which]
+        out = np.empty((c.n_layers, width), np.uint16)
+        lib().llama3_read_fused_vectors(self.cache, which, out.ctypes.data)
+        return out
+
     def set_sampling(self, on):
         """inference() returns the reference's temperature/top-k/top-p sample (True) or the argmax (False)."""
         lib().llama3_set_sampling(self.cache, 1 if on else 0)

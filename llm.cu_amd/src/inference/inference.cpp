@@ -52,6 +52,13 @@ struct Engine {
     int32_t *d_pos = nullptr;    // tokens cached so far; d_tokens[*d_pos] is the next input
     int32_t *d_token = nullptr;  // [0] last argmax, [1] waits of the fused attention + projection launch that gave up
     llm_half *ao_ring = nullptr; // one attention-output buffer per layer for llm_attn_decode_rope_oproj (null: not used)
+    // the whole decode token in one launch (llm_decode_fused), when the shapes and the device allow it
+    bool fused_ok = false, fused_on = false; // measured slower than one launch per operation: opt-in
+    llm_decode_desc fdesc = {};
+    llm_decode_layer *flayers = nullptr; // device array, rebuilt when the model changes
+    llm_half *fring[2] = {nullptr, nullptr};
+    void *fcand = nullptr;
+    int fset = 0; // buffer set of the next launch
     void *ws_attn = nullptr, *ws_lm = nullptr;
     llm_half *trace_dev = nullptr;
     size_t trace_rows = 0;
@@ -65,7 +72,8 @@ struct Engine {
     bool sampling = false; // inference() samples like the reference instead of returning the argmax
     // one captured decode step per attention form: [0] single launch (up to 512 cached positions),
     // [1] span + merge launches (beyond)
-    llm_graph_t graph[2] = {nullptr, nullptr};
+    // [2], [3]: the one-launch token working in buffer set 0 / 1
+    llm_graph_t graph[4] = {nullptr, nullptr, nullptr, nullptr};
     bool long_attn = false; // form used by the next decode step that is issued
     // scratch of llama3_decode_batch (allocated by the first call on this cache as sequence 0)
     int batch_cap = 0;
@@ -127,11 +135,31 @@ void check_shapes(const Llama3 *m, const ModelConfig &c) {
 }
 
 void drop_graph(Engine *e) {
-    for (int f = 0; f < 2; ++f) {
+    for (int f = 0; f < 4; ++f) {
         if (!e->graph[f]) continue;
         llm_graph_destroy(e->graph[f]);
         e->graph[f] = nullptr;
     }
+}
+
+// Device table of per-layer pointers for llm_decode_fused; false when the q, k, v matrices of a layer
+// are not adjacent in memory (the one-launch token reads them as one matrix).
+bool build_fused_layers(Engine *e, const Llama3 *m) {
+    const ModelConfig &c = e->cfg;
+    const size_t qd = (size_t)c.n_heads * c.head_dim, kvd = (size_t)c.n_kv_heads * c.head_dim, d = c.d_model;
+    std::vector<llm_decode_layer> t(c.n_layers);
+    for (int l = 0; l < c.n_layers; ++l) {
+        const LayerW w = layer_w(m, l);
+        if (!(w.wk == w.wq + qd * d && w.wv == w.wk + kvd * d)) return false;
+        t[l] = {w.in_ln, w.wq, w.wo, w.post_ln, w.wg, w.wu, w.wd, e->kc + (size_t)l * e->kv_layer_elems,
+                e->vc + (size_t)l * e->kv_layer_elems};
+    }
+    if (!e->flayers) e->flayers = dmalloc<llm_decode_layer>(c.n_layers, "llm_malloc(layer table)");
+    llama3_check(llm_memcpy_h2d(e->flayers, t.data(), sizeof(llm_decode_layer) * t.size(), nullptr), "H2D layer table");
+    e->fdesc.embed_dev = m->embed_tokens->d_fp16_tensor;
+    e->fdesc.final_gain_dev = m->norm->d_fp16_tensor;
+    e->fdesc.lm_head_dev = m->lm_head->d_fp16_tensor;
+    return true;
 }
 
 // The captured decode graphs hold the weight pointers of the model they were captured with.  A call
@@ -144,6 +172,10 @@ void bind_model(Engine *e, const Llama3 *m) {
     drop_graph(e);
     e->model = m;
     e->model_slab = slab;
+    if (e->fring[0]) {
+        llama3_check(llm_stream_sync(e->stream), "stream sync"); // nothing in flight reads the old table
+        e->fused_ok = build_fused_layers(e, m);
+    }
 }
 
 // Issues one pass over T rows on the engine's stream.  With dev_pos the row
@@ -303,7 +335,36 @@ void capture_decode_graph(Engine *e, const Llama3 *m, int form) {
 
 // pos: position of the token this step processes (known on the host although the kernels read it
 // from device memory), which selects the attention form
+// The whole token in one launch plus the argmax reduction, in buffer set `set`.
+void issue_fused_step(Engine *e, int set) {
+    llama3_check(llm_decode_fused(&e->fdesc, e->flayers, e->fring[set], e->fring[1 - set], 0, llm_decode_fused_phases(&e->fdesc),
+                                  e->d_token + 1, e->stream),
+                 "llm_decode_fused");
+    llama3_check(llm_argmax_finish(e->fcand, llm_decode_fused_candidates(&e->fdesc), e->d_token, e->d_tokens, e->d_pos,
+                                   e->stream),
+                 "llm_argmax_finish");
+}
+
+void capture_fused_graph(Engine *e, int set) {
+    llm_graph_t &g = e->graph[2 + set];
+    if (g) return;
+    llama3_check(llm_graph_capture_begin(e->stream), "graph capture begin");
+    issue_fused_step(e, set);
+    llama3_check(llm_graph_capture_end(e->stream, &g), "graph capture end");
+}
+
 void launch_decode_step(Engine *e, const Llama3 *m, int pos) {
+    if (pos < LONG_ATTN_FROM && e->fused_ok && e->fused_on) {
+        const int set = e->fset;
+        e->fset ^= 1; // consecutive tokens alternate the hand-over buffer sets
+        if (e->use_graph) {
+            capture_fused_graph(e, set);
+            llama3_check(llm_graph_launch(e->graph[2 + set], e->stream), "graph launch");
+        } else {
+            issue_fused_step(e, set);
+        }
+        return;
+    }
     const int form = pos >= LONG_ATTN_FROM ? 1 : 0;
     if (e->use_graph) {
         capture_decode_graph(e, m, form);
@@ -391,6 +452,22 @@ extern "C" CudaCache *init_cache_cfg(Llama3 *m, const ModelConfig *cfg) {
     }
     llama3_check(llm_fill_zero(e->d_tokens, sizeof(int32_t) * (R + 1), e->stream), "zero tokens");
     llama3_check(llm_fill_zero(e->d_pos, sizeof(int32_t), e->stream), "zero pos");
+    {
+        llm_decode_desc &f = e->fdesc;
+        f.n_layers = c.n_layers, f.d_model = d, f.n_heads = c.n_heads, f.n_kv_heads = c.n_kv_heads, f.head_dim = c.head_dim;
+        f.ffn_dim = c.ffn_dim, f.vocab = c.vocab, f.max_pos = c.max_pos, f.rms_eps = c.rms_eps;
+        f.rope_table_dev = e->rope_table, f.pos_dev = e->d_pos, f.tokens_dev = e->d_tokens, f.logits_dev = e->logits;
+        if (llm_decode_fused_supported(&f)) {
+            const size_t halves = llm_decode_fused_ring_halves(&f);
+            for (int i = 0; i < 2; ++i) {
+                e->fring[i] = dmalloc<llm_half>(halves, "llm_malloc(hand-over buffers)");
+                llama3_check(llm_attn_oproj_buffer_init(e->fring[i], (int)halves, e->stream), "arm hand-over buffers");
+            }
+            e->fcand = dmalloc<uint64_t>((size_t)llm_decode_fused_candidates(&f), "llm_malloc(argmax candidates)");
+            f.candidates_dev = e->fcand;
+            e->fused_ok = build_fused_layers(e, m);
+        }
+    }
     size_t wa = llm_attn_decode_workspace_bytes(c.n_heads, c.head_dim);
     wa = (wa + 3) / 4 * 4;
     llama3_check(llm_malloc(&e->ws_attn, wa), "llm_malloc(attention workspace)");
@@ -441,7 +518,7 @@ extern "C" void free_cache(CudaCache *C) {
         llm_stream_sync(e->stream);
         drop_graph(e);
         void *bufs[] = {e->x, e->xn, e->qkv, e->attn, e->ffn, e->logits, e->kc, e->vc, e->rope_table,
-                        e->d_tokens, e->d_pos, e->d_token, e->ao_ring, e->ws_attn, e->ws_lm, e->trace_dev, e->inject_dev,
+                        e->d_tokens, e->d_pos, e->d_token, e->ao_ring, e->flayers, e->fring[0], e->fring[1], e->fcand, e->ws_attn, e->ws_lm, e->trace_dev, e->inject_dev,
                         e->b_logits, e->b_ids, e->b_ws_attn, e->b_ws_argmax};
         for (void *b : bufs) llm_free(b);
         for (auto ev : e->ev) llm_event_destroy(ev);
@@ -504,7 +581,13 @@ extern "C" int llama3_generate(Llama3 *m, CudaCache *C, const int *prompt, int n
     // capture outside the timed decode region
     if (e->use_graph && n_decode > 1) {
         const int first_pos = start + n_prompt, last_pos = start + n_prompt + n_decode - 2;
-        if (first_pos < LONG_ATTN_FROM) capture_decode_graph(e, m, 0);
+        if (first_pos < LONG_ATTN_FROM) {
+            if (e->fused_ok && e->fused_on) {
+                capture_fused_graph(e, 0);
+                capture_fused_graph(e, 1);
+            }
+            if (!(e->fused_ok && e->fused_on) || last_pos >= LONG_ATTN_FROM) capture_decode_graph(e, m, 0);
+        }
         if (last_pos >= LONG_ATTN_FROM) capture_decode_graph(e, m, 1);
     }
     llama3_check(llm_event_record(e->ev[2], s), "event record");
@@ -641,6 +724,28 @@ extern "C" void llama3_read_logits(CudaCache *C, llm_half *logits) {
     llama3_check(llm_memcpy_d2h(logits, e->logits, sizeof(llm_half) * (size_t)e->cfg.vocab, e->stream), "D2H logits");
     llama3_check(llm_stream_sync(e->stream), "stream sync");
 }
+
+// Vectors that the last one-launch decode token handed over between its phases, for every layer:
+// which = 0 qkv, 1 attention output, 2 x after the O projection, 3 FFN hidden vector, 4 x after the down
+// projection (the layer's output).  out: [n_layers][width of that vector] fp16.
+extern "C" void llama3_read_fused_vectors(CudaCache *C, int which, llm_half *out) {
+    Engine *e = eng(C);
+    if (!e->fring[0] || which < 0 || which > 4) llama3_fail("llama3_read_fused_vectors: no one-launch token has run");
+    const ModelConfig &c = e->cfg;
+    const size_t qd = (size_t)c.n_heads * c.head_dim, qkv = qd + 2 * (size_t)c.n_kv_heads * c.head_dim, d = c.d_model;
+    const size_t F = c.ffn_dim, per_layer = qkv + qd + 2 * d + F;
+    const size_t off[5] = {0, qkv, qkv + qd, qkv + qd + d, qkv + qd + d + F}, width[5] = {qkv, qd, d, F, d};
+    const llm_half *set = e->fring[e->fset ^ 1]; // the set the last launch worked in
+    for (int l = 0; l < c.n_layers; ++l)
+        llama3_check(llm_memcpy_d2h(out + (size_t)l * width[which], set + per_layer * l + off[which],
+                                    sizeof(llm_half) * width[which], e->stream),
+                     "D2H hand-over vector");
+    llama3_check(llm_stream_sync(e->stream), "stream sync");
+}
+
+extern "C" void llama3_set_fused_decode(CudaCache *C, int on) { eng(C)->fused_on = on != 0; }
+
+extern "C" int llama3_fused_decode_active(const CudaCache *C) { return eng(C)->fused_ok && eng(C)->fused_on; }
 
 extern "C" void llama3_set_use_graph(CudaCache *C, int on) {
     Engine *e = eng(C);

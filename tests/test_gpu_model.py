@@ -175,6 +175,48 @@ def test_cache_follows_a_change_of_model(gpu):
     m2.close()
 
 
+@pytest.mark.parametrize("name,over,n_prompt,n_decode", [("tiny", dict(max_pos=128), 20, 40),
+                                                        ("tiny", dict(max_pos=1024), 490, 40),
+                                                        ("8b", dict(n_layers=2, max_pos=256), 33, 24),
+                                                        ("8b", dict(n_layers=3, max_pos=128), 7, 12)])
+def test_one_launch_token_equals_one_launch_per_operation(gpu, name, over, n_prompt, n_decode):
+    """llm_decode_fused (the whole decode token in one launch, vectors handed over inside the kernel) against
+    the per-operation launches: same greedy ids and, after every step, the same logits bit for bit; with and
+    without graph replay, through llama3_generate and through llama3_decode; the prompt of the second tiny
+    case ends at position 490, so its steps cross position 512 where the long-context kernels take over."""
+    cfg = gpu.engine.config(name, **over)
+    model = gpu.engine.Model.seeded(cfg, 61).to_device()
+    prompt = gpu.engine.seeded_tokens(61, n_prompt, cfg.vocab)
+    ref = gpu.engine.Engine(model, cfg, use_graph=False)
+    assert not ref.fused_decode_active   # opt-in: one launch per operation is the default (and the faster path)
+    want, _ = ref.generate(prompt, n_decode)
+    for use_graph in (True, False):
+        eng = gpu.engine.Engine(model, cfg, use_graph=use_graph)
+        eng.set_fused_decode(True)
+        assert eng.fused_decode_active
+        got, _ = eng.generate(prompt, n_decode)
+        assert list(got) == list(want), use_graph
+        assert np.array_equal(eng.logits(), ref.logits())
+        eng.reset()
+        got2, _ = eng.generate(prompt, n_decode)   # the hand-over buffers are back in their armed state
+        assert list(got2) == list(want)
+        eng.close()
+    # step by step, logits compared after every token
+    eng = gpu.engine.Engine(model, cfg, use_graph=True)
+    eng.set_fused_decode(True)
+    ref.reset()
+    t_e, _ = eng.prefill(prompt)
+    t_r, _ = ref.prefill(prompt)
+    for step in range(min(n_decode, 12)):
+        assert t_e == t_r
+        t_e, _ = eng.decode(t_e)
+        t_r, _ = ref.decode(t_r)
+        assert np.array_equal(eng.logits(), ref.logits()), step
+    eng.close()
+    ref.close()
+    model.close()
+
+
 def test_decode_across_the_long_context_attention_switch(gpu):
     """Greedy decoding from position 500 to 560 changes attention kernels at 512 cached positions (one
     launch before, span + merge launches after) and graphs with them: same ids with and without graphs,
