@@ -27,13 +27,31 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK = 8.0e12          # B/s, MI355X HBM3E
-# HBM bytes one launch of the gate/up SwiGLU GEMV moves, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE
-# (two runs of this script), each scaled by the same counter's reading for the calibration copy of
-# kernel_roofline() (FETCH_SIZE reads 0.5001 of the bytes a plain streaming pass fetches on this part,
-# WRITE_SIZE 1.0000): 234,985,724 fetched + 114,697 written; profiles/gemv_swiglu_hbm_traffic.md holds
-# the counter readings.
-GEMV_SWIGLU_TRAFFIC_BYTES = 235100421
 MFMA_F16_PEAK = 2.5e15     # flop/s, MI355X dense fp16
+# HBM bytes one launch of the gate/up SwiGLU GEMV moves, from two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE) of
+# this script, each scaled by the same counter's reading for the calibration copy of kernel_roofline(): kept in a
+# small file beside the counter summary, together with the git blob hashes of the kernel sources it was measured
+# at.  When a source has changed since, the figure is stale and is not reported.
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "gemv_swiglu_hbm_traffic.json")
+
+
+def blob_hash(path):
+    """git's blob hash of a file (sha1 over 'blob <size>\\0' + content), without needing git."""
+    import hashlib
+    data = open(path, "rb").read()
+    return hashlib.sha1(b"blob %d\0" % len(data) + data).hexdigest()
+
+
+def measured_traffic():
+    """(bytes or None, note) for roofline.traffic."""
+    try:
+        t = json.load(open(TRAFFIC_FILE))
+    except (OSError, ValueError):
+        return None, "no counter measurement on file"
+    for rel, want in t.get("sources", {}).items():
+        if blob_hash(os.path.join(ROOT, rel)) != want:
+            return None, "%s changed since the counter run: measure again" % rel
+    return int(t["traffic_bytes"]), "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a plain copy (profiles/gemv_swiglu_hbm_traffic.md)"
 
 
 def decode_bytes(ctx):
@@ -84,9 +102,8 @@ def main():
     orc_w = None
     if not a.no_cpu_baseline:
         from oracle import pyoracle as orc
-        from tests import helpers as H
         t0 = time.time()
-        orc_w = H.oracle_weights(model)  # fp16 copies for the CPU port, before to_cuda frees the bf16
+        orc_w = orc.weights_from_bf16(model.host_bf16())  # fp16 copies for the CPU port, before to_cuda frees the bf16
         log("fp16 host copy for the CPU baseline in %.1f s" % (time.time() - t0))
 
     t0 = time.time()
@@ -112,8 +129,15 @@ def main():
     log("decode: %d steps in %.2f ms -> %.1f tok/s (%.1f%% of HBM roofline), prompt pass %.2f ms, wall %.2f s"
         % (K, st.decode_ms, tok_s, 100 * frac, st.prefill_ms, wall))
 
-    # ---- dominant kernel against its roofline (HIP events on its own stream) -------------
+    # ---- the reference's own loop: tokens_to_cuda once, then inference() per token (src/main.cu:109-123) ----
+    api = inference_api_loop(pkg, model, engine, cfg, prompt, 64)
+    log("inference() per token, as the reference's main loop drives it: %.1f tok/s (%.3f of llama3_generate)"
+        % (api["tok_per_s"], api["tok_per_s"] / tok_s))
+
+    # ---- dominant kernels against their rooflines (HIP events on their own stream) -------------
     roof = kernel_roofline(pkg, model, cfg)
+    if not a.no_prefill_8k:
+        roof["prefill"] = prefill_kernel_roofline(pkg, model, cfg)
 
     # ---- 8192-token prompt pass ---------------------------------------------------------------
     prefill = None
@@ -201,7 +225,7 @@ def main():
                                "decode steps, fp16 KV cache" % (a.prompt, K),
                    "prompt_tokens": a.prompt, "decode_steps": K, "graph": not a.no_graph},
         "decode_hbm_frac": frac, "decode_bytes_per_token": decode_bytes(ctx_avg),
-        "prompt_pass_ms": st.prefill_ms,
+        "prompt_pass_ms": st.prefill_ms, "inference_api_tok_per_s": api["tok_per_s"], "inference_api": api,
         "roofline": roof, "cpu_baseline": cpu, "prefill_8k": prefill, "batched_decode": batched,
         "first_tokens": [int(t) for t in toks[:8]],
     }
@@ -222,11 +246,12 @@ def kernel_roofline(pkg, model, cfg):
     h = model.handle.contents
     wg = [h.layers[l].contents.mlp_gate_proj.contents.d_fp16_tensor for l in range(cfg.n_layers)]
     wu = [h.layers[l].contents.mlp_up_proj.contents.d_fp16_tensor for l in range(cfg.n_layers)]
+    gain = [h.layers[l].contents.post_attention_layernorm.contents.d_fp16_tensor for l in range(cfg.n_layers)]
     timer = ops.Timer()
 
-    def issue(stream):
+    def issue(stream):  # the launch the decode step uses: RMSNorm folded into the gate/up GEMV
         for l in range(cfg.n_layers):
-            pkg.capi.check(lib.llm_linear_swiglu(x.ptr, d, wg[l], wu[l], out.ptr, F, 1, F, d, stream))
+            pkg.capi.check(lib.llm_norm_linear_swiglu(x.ptr, gain[l], cfg.rms_eps, wg[l], wu[l], out.ptr, F, d, stream))
 
     ms = timer.time(issue, iters=8, warmup=2) / cfg.n_layers
     # One plain streaming pass of known size (2^26 elements: 128 MiB read, 128 MiB written) as the
@@ -240,12 +265,93 @@ def kernel_roofline(pkg, model, cfg):
     pkg.capi.sync()
     cal_in.free()
     cal_out.free()
-    alg = 2 * 2 * F * d + 2 * d + 2 * F  # two weight matrices + activation in + result out
+    alg = 2 * 2 * F * d + 2 * d + 2 * d + 2 * F  # two weight matrices + activation and gains in + result out
     achieved = alg / (ms * 1e-3)
-    return {"kernel": "gemv_swiglu_kernel (gate+up, N=14336, K=4096, T=1)", "bound": "hbm",
-            "achieved": achieved / 1e9, "peak": HBM_PEAK / 1e9, "unit": "GB/s", "frac": achieved / HBM_PEAK,
-            "traffic": GEMV_SWIGLU_TRAFFIC_BYTES, "avg_launch_us": ms * 1e3, "algorithmic_bytes_per_launch": alg,
-            "launches_timed": 8 * cfg.n_layers}
+    traffic, note = measured_traffic()
+    return {"kernel": "gemv_kernel<1> = llm_norm_linear_swiglu (RMSNorm + gate/up + SiLU*mul, N=14336, K=4096, T=1)",
+            "bound": "hbm", "achieved": achieved / 1e9, "peak": HBM_PEAK / 1e9, "unit": "GB/s",
+            "frac": achieved / HBM_PEAK, "traffic": traffic, "traffic_note": note, "avg_launch_us": ms * 1e3,
+            "algorithmic_bytes_per_launch": alg, "launches_timed": 8 * cfg.n_layers}
+
+
+def prefill_kernel_roofline(pkg, model, cfg, T=8192):
+    """The two kernels that carry the 8192-token prompt pass, timed alone with HIP events on their stream: the
+    gate/up GEMM with the SwiGLU epilogue (2 * T * 2F * d flop) and the causal GQA attention (4 * hd * Hq *
+    T * (T + 1) / 2 flop: only the keys j <= i are counted)."""
+    lib, ops = pkg.lib(), pkg.ops
+    d, F, Hq, Hkv, hd = cfg.d_model, cfg.ffn_dim, cfg.n_heads, cfg.n_kv_heads, cfg.head_dim
+    rng = np.random.default_rng(1)
+    x = pkg.capi.DevBuf.from_host(rng.standard_normal((T, d)).astype(np.float16).view(np.uint16))
+    hbuf = pkg.capi.DevBuf((T, F), np.uint16)
+    hm = model.handle.contents
+    wg = [hm.layers[l].contents.mlp_gate_proj.contents.d_fp16_tensor for l in range(cfg.n_layers)]
+    wu = [hm.layers[l].contents.mlp_up_proj.contents.d_fp16_tensor for l in range(cfg.n_layers)]
+    timer = ops.Timer()
+    n_l = min(cfg.n_layers, 8)
+
+    def gemm(stream):
+        for l in range(n_l):
+            pkg.capi.check(lib.llm_linear_swiglu(x.ptr, d, wg[l], wu[l], hbuf.ptr, F, T, F, d, stream))
+
+    ms_g = timer.time(gemm, iters=3, warmup=1) / n_l
+    fl_g = 2.0 * T * 2 * F * d
+    qkv = pkg.capi.DevBuf.from_host((0.5 * rng.standard_normal((T, (Hq + 2 * Hkv) * hd))).astype(np.float16).view(np.uint16))
+    kc = pkg.capi.DevBuf.from_host((0.5 * rng.standard_normal((Hkv, T, hd))).astype(np.float16).view(np.uint16))
+    vc = pkg.capi.DevBuf.from_host((0.5 * rng.standard_normal((Hkv, hd, T))).astype(np.float16).view(np.uint16))
+    ao = pkg.capi.DevBuf((T, Hq * hd), np.uint16)
+
+    def attn(stream):
+        pkg.capi.check(lib.llm_attn_prefill(qkv.ptr, (Hq + 2 * Hkv) * hd, kc.ptr, vc.ptr, ao.ptr, Hq * hd, T, 0, Hq, Hkv, hd,
+                                            T, stream))
+
+    ms_a = timer.time(attn, iters=8, warmup=2)
+    fl_a = 4.0 * hd * Hq * T * (T + 1) / 2
+    for b in (x, hbuf, qkv, kc, vc, ao):
+        b.free()
+    return {"kernel": "gemm_dma_kernel<2,2,2,4,true,1,4> = llm_linear_swiglu (gate/up + SiLU*mul, T=8192, N=2x14336, K=4096)",
+            "bound": "mfma", "flops": fl_g, "avg_us": ms_g * 1e3, "achieved": fl_g / (ms_g * 1e-3) / 1e12,
+            "peak": MFMA_F16_PEAK / 1e12, "unit": "TFLOP/s", "frac": fl_g / (ms_g * 1e-3) / MFMA_F16_PEAK,
+            "attention": {"kernel": "attn_prefill_kernel<128,4,2> = llm_attn_prefill (T=8192, 32/8 heads, causal)",
+                          "flops": fl_a, "avg_us": ms_a * 1e3, "achieved": fl_a / (ms_a * 1e-3) / 1e12,
+                          "frac": fl_a / (ms_a * 1e-3) / MFMA_F16_PEAK}}
+
+
+def inference_api_loop(pkg, model, engine, cfg, prompt, n_tokens):
+    """The reference's token loop (src/main.cu:109-123) against this library: tokens_to_cuda once, then one
+    inference() call per generated token on the growing token array; wall-clock per call from the second call on
+    (the first call is the prompt pass)."""
+    lib = pkg.lib()
+    engine.reset()
+    tokens = np.zeros(2049, np.int32)
+    n = len(prompt)
+    tokens[0] = n + 1
+    tokens[1:n + 1] = prompt
+    libc = C.CDLL("libc.so.6")
+    libc.malloc.restype = C.c_void_p
+    X = C.cast(libc.malloc(C.sizeof(pkg.capi.Tensor)), C.POINTER(pkg.capi.Tensor))  # _free_tensor frees it, as in main.cu
+    tp = tokens.ctypes.data_as(C.POINTER(C.c_int))
+    d_tokens = lib.tokens_to_cuda(tp, cfg.d_model, X)
+    nxt = lib.inference(model.handle, X, d_tokens, tp, engine.cache)  # prompt pass
+    out = [int(nxt)]
+    tokens[tokens[0]] = nxt
+    tokens[0] += 1
+    for _ in range(4):  # warm-up decode calls (graph capture)
+        nxt = lib.inference(model.handle, X, d_tokens, tp, engine.cache)
+        out.append(int(nxt))
+        tokens[tokens[0]] = nxt
+        tokens[0] += 1
+    t0 = time.time()
+    for _ in range(n_tokens):
+        nxt = lib.inference(model.handle, X, d_tokens, tp, engine.cache)
+        tokens[tokens[0]] = nxt
+        tokens[0] += 1
+    dt = time.time() - t0
+    lib._free_tensor(X)
+    pkg.capi.check(lib.llm_free(C.cast(d_tokens, C.c_void_p)))
+    engine.reset()
+    return {"tokens": n_tokens, "ms_per_call": 1e3 * dt / n_tokens, "tok_per_s": n_tokens / dt,
+            "what": "tokens_to_cuda once, then inference(model, X, d_tokens, h_tokens, cache) per token; each call returns "
+                    "the greedy id and leaves the fp16 logits in cache->h_token_probdist (one stream sync per call)"}
 
 
 if __name__ == "__main__":

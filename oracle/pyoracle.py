@@ -304,6 +304,25 @@ def forward_recompute(cfg, weights, tokens, want_hidden=False):
     return tok, hidden, logits
 
 
+def weights_from_bf16(h):
+    """fp16 weight dict for Model() from the host bf16 payloads of a not-yet-uploaded model (the dict
+    llm.cu_amd's engine.Model.host_bf16() returns): the oracle's own BF16->FP16 over the same bits the GPU
+    will convert."""
+    conv = lambda a: bf16_to_fp16(np.ascontiguousarray(a).reshape(-1)).reshape(a.shape)
+    return {
+        "embed": conv(h["embed"]), "lm_head": conv(h["lm_head"]), "norm": conv(h["norm"]),
+        "input_ln": [conv(a) for a in h["input_layernorm"]],
+        "post_ln": [conv(a) for a in h["post_attention_layernorm"]],
+        "wq": [conv(a) for a in h["self_attn_q_proj"]],
+        "wk": [conv(a) for a in h["self_attn_k_proj"]],
+        "wv": [conv(a) for a in h["self_attn_v_proj"]],
+        "wo": [conv(a) for a in h["self_attn_o_proj"]],
+        "wgate": [conv(a) for a in h["mlp_gate_proj"]],
+        "wup": [conv(a) for a in h["mlp_up_proj"]],
+        "wdown": [conv(a) for a in h["mlp_down_proj"]],
+    }
+
+
 def num_threads():
     return lib().orc_num_threads()
 

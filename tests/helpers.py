@@ -61,22 +61,8 @@ def cfg_dict(cfg):
 
 
 def oracle_weights(model):
-    """fp16 weights for the oracle from a host-side (not yet uploaded) Model:
-    the oracle's own BF16->FP16 over the same bf16 bits the GPU will convert."""
-    h = model.host_bf16()
-    conv = lambda a: orc.bf16_to_fp16(np.ascontiguousarray(a).reshape(-1)).reshape(a.shape)
-    return {
-        "embed": conv(h["embed"]), "lm_head": conv(h["lm_head"]), "norm": conv(h["norm"]),
-        "input_ln": [conv(a) for a in h["input_layernorm"]],
-        "post_ln": [conv(a) for a in h["post_attention_layernorm"]],
-        "wq": [conv(a) for a in h["self_attn_q_proj"]],
-        "wk": [conv(a) for a in h["self_attn_k_proj"]],
-        "wv": [conv(a) for a in h["self_attn_v_proj"]],
-        "wo": [conv(a) for a in h["self_attn_o_proj"]],
-        "wgate": [conv(a) for a in h["mlp_gate_proj"]],
-        "wup": [conv(a) for a in h["mlp_up_proj"]],
-        "wdown": [conv(a) for a in h["mlp_down_proj"]],
-    }
+    """fp16 weights for the oracle from a host-side (not yet uploaded) Model."""
+    return orc.weights_from_bf16(model.host_bf16())
 
 
 def run_model_parity(pkg, cfg, seed, n_prompt, n_decode, use_graph=True, oracle_decode=None):
