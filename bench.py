@@ -82,6 +82,8 @@ def main():
     ap.add_argument("--cpu-steps", type=int, default=8)
     ap.add_argument("--no-graph", action="store_true")
     ap.add_argument("--no-batch", action="store_true")
+    ap.add_argument("--ceiling", action="store_true",
+                    help="instead of the benchmark: MFMA-only probe and the 8192-token pass with amd-smi power/clock samples")
     a = ap.parse_args()
     if a.gpus != 1:
         sys.exit("bench.py: this build measures one MI355X; --gpus %d is not supported "
@@ -92,6 +94,8 @@ def main():
     pkg.init(0)
     lib = pkg.lib()
     eng_mod = pkg.engine
+    if a.ceiling:
+        return power_ceiling(pkg, a)
 
     cfg = eng_mod.config("8b", max_pos=8704)
     t0 = time.time()
@@ -230,6 +234,100 @@ def main():
         "first_tokens": [int(t) for t in toks[:8]],
     }
     print(json.dumps(out), flush=True)
+
+
+class SmiSampler:
+    """amd-smi power and shader clocks, polled from a thread while something runs on the GPU."""
+
+    def __init__(self):
+        import threading
+        self.samples, self._stop = [], threading.Event()
+        self._t = threading.Thread(target=self._run, daemon=True)
+
+    def _run(self):
+        import subprocess
+        while not self._stop.is_set():
+            try:
+                out = subprocess.run(["amd-smi", "metric", "--power", "--clock", "--json"], capture_output=True, text=True,
+                                     timeout=5).stdout
+                g = json.loads(out)["gpu_data"][0]
+                clk = [v["clk"]["value"] for k, v in g["clock"].items() if k.startswith("gfx_") and isinstance(v["clk"], dict)]
+                self.samples.append((time.time(), float(g["power"]["socket_power"]["value"]), sum(clk) / max(len(clk), 1)))
+            except Exception as e:  # the tool is optional: no samples, no figure
+                self.samples.append((time.time(), float("nan"), float("nan")))
+                time.sleep(0.2)
+
+    def __enter__(self):
+        self._t.start()
+        return self
+
+    def __exit__(self, *exc):
+        self._stop.set()
+        self._t.join()
+
+    def window(self, t0, t1):
+        w = [(p, c) for t, p, c in self.samples if t0 + 0.15 <= t <= t1 and p == p]
+        if not w:
+            return {"samples": 0}
+        return {"samples": len(w), "power_w_mean": sum(p for p, _ in w) / len(w), "power_w_max": max(p for p, _ in w),
+                "gfx_clk_mhz_mean": sum(c for _, c in w) / len(w), "gfx_clk_mhz_min": min(c for _, c in w)}
+
+
+def power_ceiling(pkg, a):
+    """What the board's power limit leaves of the 2.5 PFLOP/s fp16 figure: nothing but MFMAs with constant and with
+    random operands, then the 8192-token prompt pass and its gate/up GEMM, each for a second or more with amd-smi
+    sampled alongside.  Prints one JSON object."""
+    lib, eng_mod = pkg.lib(), pkg.engine
+    res = {}
+    with SmiSampler() as smi:
+        time.sleep(1.0)
+        res["idle"] = smi.window(time.time() - 1.0, time.time())
+        for kind, name in ((0, "mfma_only_constant_operands"), (1, "mfma_only_random_operands")):
+            tf, ms = C.c_double(0), C.c_float(0)
+            t0 = time.time()
+            pkg.capi.check(lib.llm_mfma_probe(kind, C.c_float(2500.0), C.byref(tf), C.byref(ms), None))
+            res[name] = dict(tflops=tf.value, frac_of_2500=tf.value / 2500.0, ms=ms.value, **smi.window(t0, time.time()))
+            log(name, res[name])
+            time.sleep(1.0)
+        cfg = eng_mod.config("8b", max_pos=8192)
+        model = eng_mod.Model.seeded(cfg, a.seed).to_device()
+        engine = eng_mod.Engine(model, cfg)
+        p8k = eng_mod.seeded_tokens(a.seed + 1, 8192, cfg.vocab)
+        engine.generate(p8k, 1)
+        time.sleep(1.0)
+        t0 = time.time()
+        passes = []
+        for _ in range(12):
+            engine.reset()
+            _, st8 = engine.generate(p8k, 1)
+            passes.append(st8.prefill_ms)
+        ms8 = sorted(passes)[len(passes) // 2]
+        res["prefill_8192"] = dict(ms=ms8, tflops=prefill_flops(8192) / (ms8 * 1e-3) / 1e12,
+                                   frac_of_2500=prefill_flops(8192) / (ms8 * 1e-3) / MFMA_F16_PEAK, **smi.window(t0, time.time()))
+        log("prefill_8192", res["prefill_8192"])
+        time.sleep(1.0)
+        # the gate/up GEMM alone, back to back for about two seconds
+        d, F, T = cfg.d_model, cfg.ffn_dim, 8192
+        x = pkg.capi.DevBuf.from_host(np.random.default_rng(1).standard_normal((T, d)).astype(np.float16).view(np.uint16))
+        hb = pkg.capi.DevBuf((T, F), np.uint16)
+        hm = model.handle.contents
+        wg = [hm.layers[l].contents.mlp_gate_proj.contents.d_fp16_tensor for l in range(cfg.n_layers)]
+        wu = [hm.layers[l].contents.mlp_up_proj.contents.d_fp16_tensor for l in range(cfg.n_layers)]
+        timer = pkg.ops.Timer()
+
+        def gemm(stream):
+            for l in range(cfg.n_layers):
+                pkg.capi.check(lib.llm_linear_swiglu(x.ptr, d, wg[l], wu[l], hb.ptr, F, T, F, d, stream))
+
+        t0 = time.time()
+        ms_g = timer.time(gemm, iters=36, warmup=2) / cfg.n_layers
+        fl = 2.0 * T * 2 * F * d
+        res["gate_up_gemm_8192"] = dict(us=ms_g * 1e3, tflops=fl / (ms_g * 1e-3) / 1e12, frac_of_2500=fl / (ms_g * 1e-3) / MFMA_F16_PEAK,
+                                        **smi.window(t0, time.time()))
+        log("gate_up_gemm_8192", res["gate_up_gemm_8192"])
+        engine.close()
+        model.close()
+    print(json.dumps(res), flush=True)
 
 
 def kernel_roofline(pkg, model, cfg):

@@ -219,6 +219,13 @@ int llm_attn_prefill(const uint16_t *q_dev, int ldq, const uint16_t *k_cache_dev
                      const uint16_t *v_cache_dev, uint16_t *out_dev, int ldo, int T, int pos0,
                      int n_heads, int n_kv_heads, int head_dim, int max_pos, llm_stream_t stream);
 
+/* ---- measurement aid ---------------------------------------------------------------------------- */
+/* No counterpart in the reference.  Runs nothing but v_mfma_f32_32x32x16_f16 on every CU for about
+ * ms_target milliseconds and reports the sustained rate: kind 0 with constant operands, kind 1 with
+ * operands distributed like the prompt pass's (N(0,1) activations, N(0,0.02) weights).  The second is
+ * the ceiling that the power limit of the board leaves to the prompt-pass GEMMs. */
+int llm_mfma_probe(int kind, float ms_target, double *tflops, float *ms_out, llm_stream_t stream);
+
 /* ---- one decode token in one launch ------------------------------------------------------------- */
 /* Replaces, for positions below 512, the whole chain that inference() issues for one new token
  * (src/inference/inference.cu:149-193 at T = 1: embedding, 32 x {norm, QKV, RoPE, attention, O, +res,

@@ -138,6 +138,7 @@ HIP_ABI = {
     "llm_attn_decode_noalloc_max_bytes": (_sz, []),
     "llm_attn_decode_noalloc": (_i, [_vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _i, _vp]),
     "llm_attn_prefill": (_i, [_vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp]),
+    "llm_mfma_probe": (_i, [_i, C.c_float, C.POINTER(C.c_double), C.POINTER(C.c_float), _vp]),
     "llm_decode_fused_supported": (_i, [C.POINTER(DecodeDesc)]),
     "llm_decode_fused_ring_halves": (_sz, [C.POINTER(DecodeDesc)]),
     "llm_decode_fused_candidates": (_i, [C.POINTER(DecodeDesc)]),

@@ -1,0 +1,96 @@
+// Measurement aid, not part of the token loop: what the matrix pipes of this part sustain when nothing but
+// MFMAs run, with operands of a chosen kind.  The dense fp16 peak (2.5 PFLOP/s) assumes the full clock; under the
+// board's power limit the sustained rate depends on how many operand bits toggle, so the ceiling that the
+// prompt-pass GEMMs can be held against is this probe's figure for operands distributed like theirs.
+#include <hip/hip_runtime.h>
+
+#include "common.hpp"
+
+// Every wavefront: `iters` rounds of sixteen v_mfma_f32_32x32x16_f16 over four A and four B operand sets (every
+// MFMA sees operands that differ from its predecessor's, as in a GEMM) into eight accumulators (128 accumulator
+// registers, no dependency stalls).  kind 0: all operands 1.0; kind 1: normal(0, 1) activations against
+// normal(0, 0.02) weights from a counter-based generator, different in every lane and set.
+__global__ __launch_bounds__(256) void mfma_probe_kernel(float *sink, int iters, int kind) {
+    half8_t a[4], b[4];
+    float16_t acc[8];
+    const unsigned id = blockIdx.x * blockDim.x + threadIdx.x;
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            if (kind == 0) {
+                a[p][i] = (half_t)1.0f;
+                b[p][i] = (half_t)1.0f;
+            } else {
+                // two hashes -> Box-Muller
+                unsigned h1 = (id * 32u + p * 8u + i) * 2654435761u + 12345u, h2 = h1 * 1664525u + 1013904223u;
+                h1 ^= h1 >> 15, h1 *= 2246822519u, h1 ^= h1 >> 13;
+                h2 ^= h2 >> 16, h2 *= 3266489917u, h2 ^= h2 >> 15;
+                const float u1 = ((h1 >> 8) + 1) * (1.0f / 16777217.0f), u2 = (h2 >> 8) * (1.0f / 16777216.0f);
+                const float r = sqrtf(-2.0f * logf(u1));
+                a[p][i] = (half_t)(r * cosf(6.2831853f * u2));
+                b[p][i] = (half_t)(0.02f * r * sinf(6.2831853f * u2));
+            }
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[j][e] = 0.f;
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int j = 0; j < 16; ++j)
+            acc[j & 7] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[j & 3], b[(j >> 2) & 3], acc[j & 7], 0, 0, 0);
+    }
+    float s = 0.f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) s += acc[j][e];
+    if (s == 123.456f) sink[0] = s; // keeps the loop alive
+}
+
+extern "C" {
+
+// Runs the probe for about `ms_target` milliseconds on `stream` and returns the sustained rate.
+// kind: 0 constant operands, 1 random operands shaped like the prompt pass's (N(0,1) x N(0,0.02)).
+int llm_mfma_probe(int kind, float ms_target, double *tflops, float *ms_out, llm_stream_t stream) {
+    LLM_REQUIRE(tflops && (kind == 0 || kind == 1) && ms_target > 0.f, "llm_mfma_probe: arguments");
+    int cus = 0;
+    int rc = llm_cu_count_cached(&cus);
+    if (rc != LLM_OK) return rc;
+    float *sink = nullptr;
+    LLM_HIP_CHECK(hipMalloc((void **)&sink, 4));
+    hipEvent_t e0, e1;
+    LLM_HIP_CHECK(hipEventCreate(&e0));
+    LLM_HIP_CHECK(hipEventCreate(&e1));
+    hipStream_t s = (hipStream_t)stream;
+    const int grid = cus * 2; // 8 wavefronts per CU, two per SIMD
+    auto run = [&](int iters, float *ms) -> int {
+        LLM_HIP_CHECK(hipEventRecord(e0, s));
+        mfma_probe_kernel<<<dim3(grid), dim3(256), 0, s>>>(sink, iters, kind);
+        LLM_LAUNCH_CHECK("mfma_probe_kernel");
+        LLM_HIP_CHECK(hipEventRecord(e1, s));
+        LLM_HIP_CHECK(hipEventSynchronize(e1));
+        LLM_HIP_CHECK(hipEventElapsedTime(ms, e0, e1));
+        return LLM_OK;
+    };
+    float ms = 0.f;
+    int iters = 10000;
+    rc = run(iters, &ms); // calibration (and warm-up)
+    if (rc != LLM_OK) return rc;
+    double want = (double)iters * ms_target / (ms > 0.01f ? ms : 0.01f);
+    if (want > 2.0e8) want = 2.0e8;
+    iters = want < 1000 ? 1000 : (int)want;
+    rc = run(iters, &ms);
+    if (rc != LLM_OK) return rc;
+    const double flops = (double)grid * 4 /*wavefronts*/ * iters * 16.0 * (2.0 * 32 * 32 * 16);
+    *tflops = flops / (ms * 1e-3) / 1e12;
+    if (ms_out) *ms_out = ms;
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    (void)hipFree(sink);
+    return LLM_OK;
+}
+
+} // extern "C"
