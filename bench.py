@@ -135,6 +135,8 @@ def main():
 
     # ---- the reference's own loop: tokens_to_cuda once, then inference() per token (src/main.cu:109-123) ----
     api = inference_api_loop(pkg, model, engine, cfg, prompt, 64)
+    api["sampling_candidates_on_device"] = inference_api_loop(pkg, model, engine, cfg, prompt, 64, "device")
+    api["sampling_on_host"] = inference_api_loop(pkg, model, engine, cfg, prompt, 64, "host")
     log("inference() per token, as the reference's main loop drives it: %.1f tok/s (%.3f of llama3_generate)"
         % (api["tok_per_s"], api["tok_per_s"] / tok_s))
 
@@ -414,12 +416,16 @@ def prefill_kernel_roofline(pkg, model, cfg, T=8192):
                           "frac": fl_a / (ms_a * 1e-3) / MFMA_F16_PEAK}}
 
 
-def inference_api_loop(pkg, model, engine, cfg, prompt, n_tokens):
+def inference_api_loop(pkg, model, engine, cfg, prompt, n_tokens, sampling=None):
     """The reference's token loop (src/main.cu:109-123) against this library: tokens_to_cuda once, then one
     inference() call per generated token on the growing token array; wall-clock per call from the second call on
-    (the first call is the prompt pass)."""
+    (the first call is the prompt pass).  sampling: None = greedy ids; "device" / "host" = the reference's
+    sampler (temperature 0.7, top-k 50, top-p 0.9) with the candidates selected on the device / everything
+    on the host."""
     lib = pkg.lib()
     engine.reset()
+    engine.set_sampling(sampling is not None)
+    engine.set_device_sampling(sampling != "host")
     tokens = np.zeros(2049, np.int32)
     n = len(prompt)
     tokens[0] = n + 1
@@ -447,6 +453,10 @@ def inference_api_loop(pkg, model, engine, cfg, prompt, n_tokens):
     lib._free_tensor(X)
     pkg.capi.check(lib.llm_free(C.cast(d_tokens, C.c_void_p)))
     engine.reset()
+    engine.set_sampling(False)
+    engine.set_device_sampling(True)
+    if sampling is not None:
+        return {"tokens": n_tokens, "ms_per_call": 1e3 * dt / n_tokens, "tok_per_s": n_tokens / dt}
     return {"tokens": n_tokens, "ms_per_call": 1e3 * dt / n_tokens, "tok_per_s": n_tokens / dt,
             "what": "tokens_to_cuda once, then inference(model, X, d_tokens, h_tokens, cache) per token; each call returns "
                     "the greedy id and leaves the fp16 logits in cache->h_token_probdist (one stream sync per call)"}

@@ -156,6 +156,17 @@ int llama3_sample_with(int vocab, float temperature, int top_k, float top_p, flo
 /* inference() returns the greedy id (0, default) or sample_next_token() of the logits as the
  * reference does (1). */
 void llama3_set_sampling(CudaCache *c, int on);
+/* With sampling on and settings under which only the k most probable ids can be drawn (0 < top_k <
+ * vocab, 0 < top_p <= 0.99), the exponentials' sum and the k candidates are computed on the device
+ * (llm_sample_candidates) and the host draws from k pairs instead of exponentiating, normalising and
+ * ordering the vocabulary; the ids drawn are those of sample_next_token() for the same rand() stream.
+ * f_token_probdist is then not written.  0 turns this off (every draw on the host); default 1.  The
+ * counts say how many draws of this cache went which way (the device hands a draw back when a logit is
+ * NaN, an exponential or their sum overflows, or the sum is zero). */
+void llama3_set_device_sampling(CudaCache *c, int on);
+void llama3_sampler_draw_counts(const CudaCache *c, long *device_draws, long *host_draws);
+/* The cache's sampler (settings, device selection) applied to fp16 logits [vocab] in device memory. */
+int llama3_sample_device_logits(CudaCache *c, const llm_half *logits_dev);
 /* 1: decode steps below 512 cached positions run as one launch per token (llm_decode_fused) when the
  * model shapes and the device allow it; 0 (default): one launch per operation.  Same results bit for
  * bit; on MI355X the per-operation launches are the faster of the two (305 against 361 tok/s at 8B). */

@@ -219,6 +219,28 @@ int llm_attn_prefill(const uint16_t *q_dev, int ldq, const uint16_t *k_cache_dev
                      const uint16_t *v_cache_dev, uint16_t *out_dev, int ldo, int T, int pos0,
                      int n_heads, int n_kv_heads, int head_dim, int max_pos, llm_stream_t stream);
 
+/* ---- sampler candidates --------------------------------------------------------------------------- */
+/* Device half of sample_next_token (src/inference/inference.cu:1030-1161): what temperature_softmax's
+ * loop and its qsort of the whole vocabulary (:1043-1072) decide for the first k entries, without moving
+ * the logits to the host.  exp_table_dev: 65536 floats, entry b = expf(fp16(b) / temperature) as the HOST
+ * computes it (the caller fills it, so that the values are the host library's, bit for bit), monotone in
+ * the logit.  out_dev: llm_sample_candidates_bytes(vocab, k) bytes, 16-byte aligned; only its first
+ * llm_sample_candidates_head_bytes(k) bytes are the result (the rest is the kernel's scratch space and
+ * need not travel to the host).  The result is four 32-bit words --
+ * the float32 denominator (the running sum of the table values in index order, rounded after every
+ * addition as the host loop rounds), the number of pairs n (k, or 0), a flag, the number of groups
+ * of 8 entries the sum had to add one by one -- and n pairs {float probability, int32 index}: the k entries that a
+ * stable descending sort by probability puts first, unordered among the larger ones, by index among those
+ * equal to the k-th.  flag != 0 (a NaN or infinite value, a zero or infinite denominator, a table that is
+ * not monotone, a wait inside the kernel that gave up): nothing was selected and the caller falls back to
+ * the host path.  1 <= k < vocab <= llm_sample_candidates_max_vocab().  Two launches (a clear of the scratch
+ * space and the selection, whose workgroups wait for one another); calls that share out_dev must not overlap. */
+size_t llm_sample_candidates_bytes(int vocab, int k);
+size_t llm_sample_candidates_head_bytes(int k);
+int llm_sample_candidates_max_vocab(void); /* larger vocabularies are rejected */
+int llm_sample_candidates(const uint16_t *logits_dev, const float *exp_table_dev, int vocab, int k,
+                          void *out_dev, llm_stream_t stream);
+
 /* ---- measurement aid ---------------------------------------------------------------------------- */
 /* No counterpart in the reference.  Runs nothing but v_mfma_f32_32x32x16_f16 on every CU for about
  * ms_target milliseconds and reports the sustained rate: kind 0 with constant operands, kind 1 with

@@ -131,6 +131,10 @@ HIP_ABI = {
     "llm_attn_oproj_supported": (_i, [_i, _i, _i, _i]),
     "llm_attn_oproj_buffer_init": (_i, [_vp, _i, _vp]),
     "llm_attn_decode_rope_oproj": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _vp, _vp, _vp, _i, _vp, _vp]),
+    "llm_sample_candidates_bytes": (_sz, [_i, _i]),
+    "llm_sample_candidates_head_bytes": (_sz, [_i]),
+    "llm_sample_candidates_max_vocab": (_i, []),
+    "llm_sample_candidates": (_i, [_vp, _vp, _i, _i, _vp, _vp]),
     "llm_attn_decode_rope_long": (_i, [_vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _vp, _vp]),
     "llm_norm_lmhead_argmax": (_i, [_vp, _vp, C.c_double, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp, _vp]),
     "llm_attn_decode_workspace_bytes": (_sz, [_i, _i]),
@@ -203,6 +207,9 @@ HOST_ABI = {
     "top_p_sampling": (_i, [_vp, C.c_float]),
     "llama3_sampler_config": (None, [_i, C.c_float, _i, C.c_float]),
     "llama3_set_sampling": (None, [_CP, _i]),
+    "llama3_set_device_sampling": (None, [_CP, _i]),
+    "llama3_sampler_draw_counts": (None, [_CP, C.POINTER(C.c_long), C.POINTER(C.c_long)]),
+    "llama3_sample_device_logits": (_i, [_CP, _vp]),
     "llama3_set_fused_decode": (None, [_CP, _i]),
     "llama3_fused_decode_active": (_i, [_CP]),
     "llama3_read_fused_vectors": (None, [_CP, _i, _vp]),

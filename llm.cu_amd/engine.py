@@ -206,6 +206,21 @@ class Engine:
         lib().llama3_read_fused_vectors(self.cache, which, out.ctypes.data)
         return out
 
+    def set_device_sampling(self, on):
+        lib().llama3_set_device_sampling(self.cache, 1 if on else 0)
+
+    def sampler_draw_counts(self):
+        """(draws decided from device-selected candidates, draws made by the host path)"""
+        d, h = C.c_long(0), C.c_long(0)
+        lib().llama3_sampler_draw_counts(self.cache, C.byref(d), C.byref(h))
+        return d.value, h.value
+
+    def sample_device_logits(self, logits):
+        """The cache's sampler on fp16 logits given as a host array (uploaded) or a DevBuf."""
+        buf = logits if isinstance(logits, capi.DevBuf) else capi.DevBuf.from_host(
+            np.ascontiguousarray(logits, dtype=np.uint16))
+        return lib().llama3_sample_device_logits(self.cache, buf.ptr)
+
     def set_sampling(self, on):
         """inference() returns the reference's temperature/top-k/top-p sample (True) or the argmax (False)."""
         lib().llama3_set_sampling(self.cache, 1 if on else 0)

@@ -136,6 +136,22 @@ def attn_decode_noalloc(q, kc, vc, ctx, n_heads, n_kv_heads, head_dim):
     return d_o.download()
 
 
+def sample_candidates(logits, exp_table, k):
+    """llm_sample_candidates.  Returns (denominator float32, flag, ranges added one by one,
+    probabilities float32[n], indices int32[n]) with n = k, or 0 when the flag is set."""
+    logits = _u16(logits).reshape(-1)
+    table = np.ascontiguousarray(exp_table, dtype=np.float32)
+    assert table.size == 65536
+    d_l, d_t = DevBuf.from_host(logits), DevBuf.from_host(table)
+    d_o = DevBuf((lib().llm_sample_candidates_bytes(logits.size, k) // 4,), np.uint32)
+    check(lib().llm_sample_candidates(d_l.ptr, d_t.ptr, logits.size, k, d_o.ptr, None))
+    o = d_o.download()
+    n = int(o[1])
+    pairs = o[4:4 + 2 * n].reshape(n, 2)
+    return (o[0:1].view(np.float32)[0], int(o[2]), int(o[3]), pairs[:, 0].copy().view(np.float32),
+            pairs[:, 1].copy().view(np.int32))
+
+
 def attn_prefill(q, kc, vc, pos0, n_heads, n_kv_heads, head_dim):
     q, kc, vc = _u16(q), _u16(kc), _u16(vc)
     T = q.shape[0]

@@ -70,6 +70,16 @@ struct Engine {
     int pos = 0;
     bool use_graph = true;
     bool sampling = false; // inference() samples like the reference instead of returning the argmax
+    // device half of the sampler (llm_sample_candidates): the host's exp table for table_temperature, the
+    // selection's output and its pinned mirror, sized for table_k pairs
+    bool device_select = true;   // use it whenever the settings allow
+    bool select_pending = false; // the step being issued also selects candidates
+    bool table_ok = false;       // the table is monotone (else every draw takes the host path)
+    float table_temperature = 0.0f;
+    int select_cap = 0;
+    float *d_exp_table = nullptr;
+    uint32_t *d_select = nullptr, *h_select = nullptr;
+    long device_draws = 0, host_draws = 0;
     // one captured decode step per attention form: [0] single launch (up to 512 cached positions),
     // [1] span + merge launches (beyond)
     // [2], [3]: the one-launch token working in buffer set 0 / 1
@@ -270,6 +280,56 @@ void check_handover(Engine *e) {
     if (e->h_stage[3] != 0) llama3_fail("attention/projection hand-over timed out %d time(s)", e->h_stage[3]);
 }
 
+// Brings the exp table and the selection buffers in line with the cache's sampler settings; false when
+// the settings or the table rule the device selection out.
+bool prepare_selection(Engine *e) {
+    const SamplerParams &sp = e->sampler;
+    if (!e->device_select || !sampler_head_suffices(sp) || sp.vocab > llm_sample_candidates_max_vocab()) return false;
+    if (!e->d_exp_table || e->table_temperature != sp.temperature) {
+        std::vector<float> table(65536);
+        e->table_ok = sampler_fill_exp_table(sp.temperature, table.data());
+        if (!e->d_exp_table) e->d_exp_table = dmalloc<float>(65536, "llm_malloc(exp table)");
+        llama3_check(llm_memcpy_h2d(e->d_exp_table, table.data(), sizeof(float) * 65536, e->stream), "H2D exp table");
+        llama3_check(llm_stream_sync(e->stream), "stream sync"); // `table` goes out of scope
+        e->table_temperature = sp.temperature;
+    }
+    if (!e->table_ok) return false;
+    if (sp.top_k > e->select_cap) {
+        if (e->d_select) llm_free(e->d_select);
+        if (e->h_select) llm_free_host(e->h_select);
+        e->d_select = (uint32_t *)dmalloc<char>(llm_sample_candidates_bytes(e->cfg.vocab, sp.top_k),
+                                                "llm_malloc(sampler candidates)");
+        void *hp = nullptr;
+        llama3_check(llm_malloc_host(&hp, llm_sample_candidates_head_bytes(sp.top_k)), "llm_malloc_host(sampler candidates)");
+        e->h_select = (uint32_t *)hp;
+        e->select_cap = sp.top_k;
+    }
+    return true;
+}
+
+// After the LM head of a step, in stream order: select the sampler's candidates from `logits` and bring
+// them to the host behind the token id.
+void enqueue_selection(Engine *e, const llm_half *logits) {
+    llama3_check(llm_sample_candidates(logits, e->d_exp_table, e->cfg.vocab, e->sampler.top_k, e->d_select, e->stream),
+                 "llm_sample_candidates");
+    llama3_check(llm_memcpy_d2h(e->h_select, e->d_select, llm_sample_candidates_head_bytes(e->sampler.top_k), e->stream),
+                 "D2H sampler candidates");
+}
+
+// The draw from what enqueue_selection brought back (after the stream sync); -1 when the device left the
+// decision to the host.
+int draw_from_selection(Engine *e) {
+    const uint32_t *h = e->h_select;
+    const int k = e->sampler.top_k;
+    if (h[2] != 0 || (int)h[1] != k) return -1;
+    std::vector<ProbIndex> head((size_t)k);
+    for (int i = 0; i < k; ++i) {
+        memcpy(&head[i].probability, &h[4 + 2 * i], sizeof(float));
+        head[i].index = (int)h[5 + 2 * i];
+    }
+    return sampler_draw_from_head(e->sampler, head.data(), k);
+}
+
 // Appends n host tokens at e->pos with one multi-row pass.  Leaves
 // d_pos = pos + n and d_tokens[pos + n] = the greedy next token.
 // logits_host (may be null): pinned host memory that receives the fp16 logits before the pass's one sync.
@@ -312,6 +372,7 @@ int run_pass(Engine *e, const Llama3 *m, const int *tokens, int n, llm_half *log
                      "D2H trace");
     if (logits_host)
         llama3_check(llm_memcpy_d2h(logits_host, e->logits, sizeof(llm_half) * (size_t)c.vocab, s), "D2H logits");
+    if (e->select_pending) enqueue_selection(e, e->logits);
     llama3_check(llm_stream_sync(s), "stream sync");
     check_handover(e);
     e->trace_host = nullptr;
@@ -398,6 +459,7 @@ int step_one(Engine *e, const Llama3 *m, int token, llm_half *logits_host) {
     llama3_check(llm_memcpy_d2h(&e->h_stage[2], e->d_token, sizeof(int32_t) * 2, s), "D2H token");
     if (logits_host)
         llama3_check(llm_memcpy_d2h(logits_host, e->logits, sizeof(llm_half) * (size_t)c.vocab, s), "D2H logits");
+    if (e->select_pending) enqueue_selection(e, e->logits);
     llama3_check(llm_stream_sync(s), "stream sync");
     check_handover(e);
     e->tokens.push_back(token);
@@ -524,6 +586,9 @@ extern "C" void free_cache(CudaCache *C) {
         for (auto ev : e->ev) llm_event_destroy(ev);
         llm_stream_destroy(e->stream);
         llm_free_host(e->h_stage);
+        if (e->h_select) llm_free_host(e->h_select);
+        if (e->d_select) llm_free(e->d_select);
+        if (e->d_exp_table) llm_free(e->d_exp_table);
         delete e;
     }
     llm_free_host(C->h_token_probdist);
@@ -779,13 +844,55 @@ extern "C" int inference(Llama3 *m, Tensor *X, int *d_tokens, int *h_tokens, Cud
     const int fresh = n - e->pos;
     // h_token_probdist holds the step's logits on return, as after the reference's compute_lm_head
     // (inference.cu:1021-1026); they travel behind the token id in the same stream, one sync per call
+    e->select_pending = e->sampling && prepare_selection(e);
     int tok = fresh == 1 ? step_one(e, m, ids[n - 1], C->h_token_probdist)
                          : run_pass(e, m, ids + e->pos, fresh, C->h_token_probdist);
-    if (e->sampling) tok = sampler_draw(e->sampler, C->f_token_probdist, C->h_token_probdist); // inference.cu:1028
+    if (e->sampling) { // sample_next_token, inference.cu:1028
+        int drawn = -1;
+        if (e->select_pending) {
+            e->select_pending = false;
+            drawn = draw_from_selection(e);
+        }
+        if (drawn >= 0) {
+            ++e->device_draws;
+        } else {
+            drawn = sampler_draw(e->sampler, C->f_token_probdist, C->h_token_probdist);
+            ++e->host_draws;
+        }
+        tok = drawn;
+    }
     return tok;
 }
 
 extern "C" void llama3_set_sampling(CudaCache *C, int on) { eng(C)->sampling = on != 0; }
+
+extern "C" void llama3_set_device_sampling(CudaCache *C, int on) { eng(C)->device_select = on != 0; }
+
+extern "C" void llama3_sampler_draw_counts(const CudaCache *C, long *device_draws, long *host_draws) {
+    if (device_draws) *device_draws = eng(C)->device_draws;
+    if (host_draws) *host_draws = eng(C)->host_draws;
+}
+
+// The cache's sampler applied to fp16 logits that already sit on the device.
+extern "C" int llama3_sample_device_logits(CudaCache *C, const llm_half *logits_dev) {
+    Engine *e = eng(C);
+    if (!logits_dev) llama3_fail("llama3_sample_device_logits: null logits");
+    int drawn = -1;
+    if (prepare_selection(e)) {
+        enqueue_selection(e, logits_dev);
+        llama3_check(llm_stream_sync(e->stream), "stream sync");
+        drawn = draw_from_selection(e);
+    }
+    if (drawn >= 0) {
+        ++e->device_draws;
+        return drawn;
+    }
+    llama3_check(llm_memcpy_d2h(C->h_token_probdist, logits_dev, sizeof(llm_half) * (size_t)e->cfg.vocab, e->stream),
+                 "D2H logits");
+    llama3_check(llm_stream_sync(e->stream), "stream sync");
+    ++e->host_draws;
+    return sampler_draw(e->sampler, C->f_token_probdist, C->h_token_probdist);
+}
 
 extern "C" void llama3_cache_sampler_config(CudaCache *C, float temperature, int top_k, float top_p) {
     Engine *e = eng(C);

@@ -107,6 +107,34 @@ int sampler_draw_reference(const SamplerParams &sp, float *tensor, const llm_hal
     return selected;
 }
 
+bool sampler_head_suffices(const SamplerParams &sp) {
+    return sp.top_k > 0 && sp.top_k < sp.vocab && sp.top_p > 0.0f && sp.top_p <= 0.99f;
+}
+
+static bool prob_before(const ProbIndex &a, const ProbIndex &b) {
+    return a.probability > b.probability || (a.probability == b.probability && a.index < b.index);
+}
+
+bool sampler_fill_exp_table(float temperature, float *table) {
+    for (uint32_t b = 0; b < 65536u; ++b) table[b] = expf(half_to_float((llm_half)b) / temperature);
+    // walk the finite patterns in value order: negative ones from the largest magnitude down, then the positive
+    float prev = -INFINITY;
+    bool monotone = true;
+    for (int i = 0; i < 2 * 0x7c00 && monotone; ++i) {
+        const uint32_t b = i < 0x7c00 ? 0x8000u + (uint32_t)(0x7bff - i) : (uint32_t)(i - 0x7c00);
+        const float v = table[b];
+        if (v != v || v < prev) monotone = false;
+        prev = v;
+    }
+    return monotone;
+}
+
+int sampler_draw_from_head(const SamplerParams &sp, ProbIndex *head, int k) {
+    std::sort(head, head + k, prob_before);
+    (void)top_k_pick(sp.vocab, head, k); // renormalises the head and consumes one rand(), result unused
+    return top_p_pick(sp.vocab, head, k, sp.top_p);
+}
+
 // Same result without sorting the vocabulary.  After the top-k pass has renormalised the first k
 // entries they sum to 1 up to rounding, so for top_p below that sum the top-p pass never looks past
 // entry k-1: only the k largest probabilities, in the order qsort leaves them, matter.  glibc's qsort
@@ -115,8 +143,7 @@ int sampler_draw_reference(const SamplerParams &sp, float *tensor, const llm_hal
 // full path for settings where the tail of the array is reachable.
 int sampler_draw(const SamplerParams &sp, float *tensor, const llm_half *half_tensor) {
     const int k = sp.top_k, vocab = sp.vocab;
-    if (k <= 0 || k >= vocab || !(sp.top_p > 0.0f) || sp.top_p > 0.99f)
-        return sampler_draw_reference(sp, tensor, half_tensor);
+    if (!sampler_head_suffices(sp)) return sampler_draw_reference(sp, tensor, half_tensor);
     // the exponentials are independent (any thread gives the same bits); their sum is taken afterwards in
     // index order, as the reference's single loop does
     const float temperature = sp.temperature;

@@ -13,3 +13,14 @@ struct SamplerParams {
 // tensor: float[vocab] scratch (left holding the probabilities), half_tensor: fp16 logits [vocab].
 int sampler_draw(const SamplerParams &sp, float *tensor, const llm_half *half_tensor);
 int sampler_draw_reference(const SamplerParams &sp, float *tensor, const llm_half *half_tensor);
+
+// The device-assisted form (llm_sample_candidates picks the head of the sorted array):
+// settings for which only the k largest probabilities can be drawn (the same condition under which
+// sampler_draw avoids the full sort)
+bool sampler_head_suffices(const SamplerParams &sp);
+// table[b] = expf(fp16(b) / temperature) for every fp16 bit pattern b, with this host's expf.  Returns
+// whether the finite entries do not decrease with the value of b (what the device selection relies on).
+bool sampler_fill_exp_table(float temperature, float *table65536);
+// The draws of sample_next_token from the k entries a stable descending sort would put first, given in
+// any order (sorted here by probability descending, index ascending).
+int sampler_draw_from_head(const SamplerParams &sp, ProbIndex *head, int k);
