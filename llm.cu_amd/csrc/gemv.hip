@@ -93,13 +93,18 @@ __global__ __launch_bounds__(GEMV_THREADS) void gemv_kernel(const GemvArgs a) {
     issue_next(1);
     // the residual of each of this wavefront's rows, asked for now: at the end of a row the value is
     // there instead of one more trip to memory behind the last weight load
-    half_t resv[4] = {(half_t)0.f, (half_t)0.f, (half_t)0.f, (half_t)0.f};
+    // (four named registers and a select chain below: an array indexed by the row counter would live in
+    // scratch memory)
+    half_t res0 = (half_t)0.f, res1 = (half_t)0.f, res2 = (half_t)0.f, res3 = (half_t)0.f;
     if (MODE == GV_PLAIN && a.res) {
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
+        auto ask = [&](int r) {
             const int row = row_base + row_step * r;
-            if (r < a.rpw && row < N) resv[r] = a.res[row];
-        }
+            return (r < a.rpw && row < N) ? a.res[row] : (half_t)0.f;
+        };
+        res0 = ask(0);
+        res1 = ask(1);
+        res2 = ask(2);
+        res3 = ask(3);
     }
     if (a.gain) {
         rms_finish<GEMV_THREADS, GEMV_NORM_R>(xr, xs, K, a.eps, red);
@@ -144,7 +149,7 @@ __global__ __launch_bounds__(GEMV_THREADS) void gemv_kernel(const GemvArgs a) {
                     if (lane == 0) {
                         half_t hres = (half_t)s0;
                         if (a.res) { // fp16(fp16(sum) + residual), the reference's add_norm on the stored projection
-                            const half_t rv = i < 4 ? resv[i < 4 ? i : 0] : a.res[row];
+                            const half_t rv = i == 0 ? res0 : i == 1 ? res1 : i == 2 ? res2 : i == 3 ? res3 : a.res[row];
                             hres = (half_t)((float)hres + (float)rv);
                         }
                         a.out[row] = hres;

@@ -24,3 +24,25 @@ def gpu(pkg):
     library or the device is missing (no CPU fallback exists)."""
     pkg.init(0)
     return pkg
+
+
+def _roctx():
+    """librocprofiler-sdk-roctx when LLM_TEST_ROCTX=1 (set for a `rocprofv3 --kernel-trace --marker-trace` run
+    of the suite, which then shows which test launched which kernel); None otherwise."""
+    if os.environ.get("LLM_TEST_ROCTX") != "1":
+        return None
+    if not hasattr(_roctx, "lib"):
+        import ctypes
+        _roctx.lib = ctypes.CDLL("librocprofiler-sdk-roctx.so")
+        _roctx.lib.roctxRangePushA.argtypes = [ctypes.c_char_p]
+    return _roctx.lib
+
+
+@pytest.fixture(autouse=True)
+def _test_as_marker_range(request):
+    lib = _roctx()
+    if lib:
+        lib.roctxRangePushA(request.node.nodeid.encode())
+    yield
+    if lib:
+        lib.roctxRangePop()
