@@ -32,7 +32,7 @@ MFMA_F16_PEAK = 2.5e15     # flop/s, MI355X dense fp16
 # this script, each scaled by the same counter's reading for the calibration copy of kernel_roofline(): kept in a
 # small file beside the counter summary, together with the git blob hashes of the kernel sources it was measured
 # at.  When a source has changed since, the figure is stale and is not reported.
-TRAFFIC_FILE = os.path.join(ROOT, "profiles", "gemv_swiglu_hbm_traffic.json")
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "decode_gemv_hbm_traffic.json")
 
 
 def blob_hash(path):
@@ -51,7 +51,7 @@ def measured_traffic():
     for rel, want in t.get("sources", {}).items():
         if blob_hash(os.path.join(ROOT, rel)) != want:
             return None, "%s changed since the counter run: measure again" % rel
-    return int(t["traffic_bytes"]), "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a plain copy (profiles/gemv_swiglu_hbm_traffic.md)"
+    return int(t["traffic_bytes"]), "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a plain copy (profiles/decode_gemv_hbm_traffic.md)"
 
 
 def decode_bytes(ctx):

@@ -67,24 +67,27 @@ def rope(buf, n_heads, head_dim, pos0=0, theta=500000.0, max_pos=None):
     return d_b.download()
 
 
-def linear(x, w, residual=None):
+def linear(x, w, residual=None, ldo=None):
+    """ldo: row stride of the output buffer in elements (default N); the columns beyond N are not returned."""
     x, w = _u16(x), _u16(w)
     T, K = x.shape
     N = w.shape[0]
-    d_x, d_w, d_o = DevBuf.from_host(x), DevBuf.from_host(w), DevBuf((T, N), np.uint16)
+    ldo = N if ldo is None else ldo
+    d_x, d_w, d_o = DevBuf.from_host(x), DevBuf.from_host(w), DevBuf((T, ldo), np.uint16)
     d_r = DevBuf.from_host(_u16(residual)) if residual is not None else None
-    check(lib().llm_linear(d_x.ptr, K, d_w.ptr, d_r.ptr if d_r else None, N, d_o.ptr, N, T, N, K, None))
-    return d_o.download()
+    check(lib().llm_linear(d_x.ptr, K, d_w.ptr, d_r.ptr if d_r else None, N, d_o.ptr, ldo, T, N, K, None))
+    return np.ascontiguousarray(d_o.download()[:, :N])
 
 
-def linear_swiglu(x, wgate, wup):
+def linear_swiglu(x, wgate, wup, ldo=None):
     x, wgate, wup = _u16(x), _u16(wgate), _u16(wup)
     T, K = x.shape
     N = wgate.shape[0]
+    ldo = N if ldo is None else ldo
     d_x, d_g, d_u = DevBuf.from_host(x), DevBuf.from_host(wgate), DevBuf.from_host(wup)
-    d_o = DevBuf((T, N), np.uint16)
-    check(lib().llm_linear_swiglu(d_x.ptr, K, d_g.ptr, d_u.ptr, d_o.ptr, N, T, N, K, None))
-    return d_o.download()
+    d_o = DevBuf((T, ldo), np.uint16)
+    check(lib().llm_linear_swiglu(d_x.ptr, K, d_g.ptr, d_u.ptr, d_o.ptr, ldo, T, N, K, None))
+    return np.ascontiguousarray(d_o.download()[:, :N])
 
 
 def kv_layout(k, v, n_kv_heads, head_dim, max_pos):

@@ -38,6 +38,18 @@ def test_convert_ragged_sizes(gpu, n):
     assert np.array_equal(gpu.ops.bf16_to_fp16(src), orc.bf16_to_fp16(src))
 
 
+def test_convert_between_unaligned_buffers(gpu):
+    """Source and destination that do not start on a 16-byte boundary take the element-wise kernel."""
+    n = 100003
+    src = np.random.default_rng(4).integers(0, 65536, size=n + 8, dtype=np.uint32).astype(np.uint16)
+    d_src, d_dst = gpu.capi.DevBuf.from_host(src), gpu.capi.DevBuf((n + 8,), np.uint16)
+    d_dst.zero()
+    gpu.capi.check(gpu.lib().llm_bf16_to_fp16(d_src.ptr + 2, d_dst.ptr + 6, n, None))
+    out = d_dst.download()
+    assert np.array_equal(out[3:3 + n], orc.bf16_to_fp16(src[1:1 + n]))
+    assert not out[:3].any() and not out[3 + n:].any()
+
+
 def test_convert_llama3_8b_ffn_tensor(gpu):
     # 4096 x 14336 seeded N(0, 0.02) bf16
     src = gpu.engine.seeded_normal_bf16(42, 7, 4096 * 14336)
@@ -182,6 +194,30 @@ def test_linear_gemm_ragged_shapes(gpu, T, K, N):
     assert e <= TIGHT
     got_r = gpu.ops.linear(x, w, residual=res)
     assert H.mixed_err(got_r, orc.add(orc.linear(x, w), res)) <= TOL
+
+
+@pytest.mark.parametrize("what,T,K,N,ldo", [
+    # output rows that are not a multiple of 8 bytes apart: the register-staged MFMA kernels (64x64 and 128x128 /
+    # 128x64 tiles) instead of the direct-to-LDS ones
+    ("linear", 100, 256, 272, 274), ("linear", 40, 256, 272, 274), ("swiglu", 100, 256, 272, 274),
+    ("swiglu", 20, 256, 48, None),
+    # 2..16 rows with K not a multiple of 1024: the skinny kernel that reads the weights through registers
+    ("linear", 8, 768, 512, None), ("swiglu", 8, 768, 512, None),
+    # gate/up with few output tiles and a long K at 64 and 128 rows: split k with the two-matrix reduction
+    ("swiglu", 64, 4096, 256, None), ("swiglu", 128, 4096, 256, None)])
+def test_kernel_families_off_the_main_paths(gpu, what, T, K, N, ldo):
+    """Shapes chosen so that every kernel family of the projections is launched by some test (the 8B shapes
+    only reach the direct-to-LDS and skinny-DMA kernels)."""
+    rng = np.random.default_rng(T + K + N)
+    x = H.bits(rng.standard_normal((T, K)))
+    w = H.bits(0.05 * rng.standard_normal((N, K), dtype=np.float32))
+    if what == "linear":
+        got, want = gpu.ops.linear(x, w, ldo=ldo), orc.linear(x, w)
+    else:
+        w2 = H.bits(0.05 * rng.standard_normal((N, K), dtype=np.float32))
+        got, want = gpu.ops.linear_swiglu(x, w, w2, ldo=ldo), orc.linear_swiglu(x, w, w2)
+    assert got.shape == (T, N)
+    assert H.mixed_err(got, want) <= TOL
 
 
 def test_split_k_linear_on_two_streams_at_once(gpu):
