@@ -3,7 +3,7 @@
 
 A "step" is one decode token through all 32 layers + LM head + argmax with
 the KV cache and every weight resident in HBM.  The workload is the full
-LLaMA3-8B decoder of BASELINE.json (seeded random-init bf16 weights converted
+LLaMA3-8B decoder (32 layers, seeded random-init bf16 weights converted
 to fp16 at load, prompt of 128 seeded ids, then K greedy decode steps).  The
 same run also measures the 8192-token prompt pass (MFMA GEMM + causal GQA
 attention), the dominant kernel (fused gate/up SwiGLU GEMV) against the HBM
