@@ -792,6 +792,204 @@ __global__ __launch_bounds__(WGM * WGN * 64, OCC) void gemm_dma_kernel(const hal
     }
 }
 
+// The 256 x 256 tile of gemm_dma_kernel<NB,2,2,4,true,1,4> with BK = 64: a tile row is 128 bytes, so every
+// lane group of a tile load fetches a whole cache line (8 rows x 128 B per wave instruction instead of 16 rows
+// x 64 B), and there is one workgroup barrier per 64 k instead of per 32.  Two LDS stages of 64 KB.  A step is
+// four sub-steps of 16 MFMAs on alternating fragment sets; the fragments of a sub-step are read during the one
+// before it.  The barrier sits between sub-steps 2 and 3: by then every wave has read the last fragments of
+// the current stage, and the next tile (issued during sub-step 3 of the previous step) must have landed; in
+// sub-step 3 the first fragments of the next tile are read and the loads of the tile after it are issued
+// into the stage that has just been released.
+#define DMA64_BK 64
+template <int NB>
+__global__ __launch_bounds__(256, 1) void gemm_dma64_kernel(const half_t *__restrict__ x, int ldx, const half_t *__restrict__ w,
+                                                            const half_t *__restrict__ w2, const half_t *res, int ldr,
+                                                            half_t *out, int ldo, int T, int N, int K, int tiles_m,
+                                                            int tiles_n) {
+    constexpr int FM = 4, WTM = 128, BM = 256, BROWS = 256, BN = BROWS / NB, FN = 4 / NB;
+    constexpr int STAGE_HALVES = (BM + BROWS) * DMA64_BK;
+    constexpr int LPT = (BM + BROWS) / 8 / 4; // 16 load instructions per wave per tile
+    constexpr int TA = BM / 8 / 4, TB1 = BN / 8 / 4;
+    static_assert(TA + NB * TB1 == LPT, "loader split");
+    extern __shared__ __attribute__((aligned(16))) half_t lds[];
+
+    const int nblk = tiles_m * tiles_n;
+    int bid = blockIdx.x;
+    {
+        const int per = nblk / 8;
+        if (per > 0 && bid < per * 8) bid = (bid % 8) * per + bid / 8;
+    }
+    constexpr int GROUP_M = 8;
+    const int group = bid / (GROUP_M * tiles_n);
+    const int first_m = group * GROUP_M;
+    const int gsz = tiles_m - first_m < GROUP_M ? tiles_m - first_m : GROUP_M;
+    const int tm = first_m + (bid % (GROUP_M * tiles_n)) % gsz;
+    const int tn = (bid % (GROUP_M * tiles_n)) / gsz;
+    const int m0 = tm * BM, n0 = tn * BN;
+
+    const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid / 64), lane = tid % 64;
+    const int wm = wave % 2, wn = wave / 2;
+
+    // loader: instruction q = wave + 4 t moves stage rows 8q .. 8q+7 (q < 32: A rows, else B rows), 128 B each;
+    // lane -> row lane/8, LDS chunk lane%8, which holds global chunk (lane%8) ^ ((row>>1)&7)
+    const __amdgpu_buffer_rsrc_t rs_x =
+        __builtin_amdgcn_make_buffer_rsrc((void *)x, 0, ((T - 1) * ldx + K) * (int)sizeof(half_t), 0x00020000);
+    const __amdgpu_buffer_rsrc_t rs_w = __builtin_amdgcn_make_buffer_rsrc((void *)w, 0, N * K * (int)sizeof(half_t), 0x00020000);
+    const __amdgpu_buffer_rsrc_t rs_w2 =
+        __builtin_amdgcn_make_buffer_rsrc((void *)(NB == 2 ? w2 : w), 0, N * K * (int)sizeof(half_t), 0x00020000);
+    uint32_t goff[16];
+#pragma unroll
+    for (int t = 0; t < LPT; ++t) {
+        const int q = wave + t * 4;
+        const int srow = q * 8 + lane / 8; // row inside the stage
+        const int gch = (lane & 7) ^ ((srow >> 1) & 7);
+        if (t < TA) {
+            int ar = m0 + srow;
+            ar = ar < T ? ar : T - 1;
+            goff[t] = (__umul24((unsigned)ar, (unsigned)ldx) + (unsigned)(gch * 8)) * 2u;
+        } else {
+            int br = n0 + (srow - BM) - (t >= TA + TB1 ? BN : 0);
+            br = br < N ? br : N - 1;
+            goff[t] = (__umul24((unsigned)br, (unsigned)K) + (unsigned)(gch * 8)) * 2u;
+        }
+    }
+    auto issue_one = [&](int kt, int t) {
+        half_t *st = lds + (kt & 1) * STAGE_HALVES;
+        const uint32_t k0 = (uint32_t)kt * DMA64_BK * 2u;
+        auto dst = DMA_LP(st + (wave + t * 4) * 8 * DMA64_BK);
+        if (t < TA) __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_x, dst, 16, goff[t], k0, 0, 0);
+        else if (t < TA + TB1) __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_w, dst, 16, goff[t], k0, 0, 0);
+        else __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_w2, dst, 16, goff[t], k0, 0, 0);
+    };
+
+    const int frow = lane % 32, sw = (frow >> 1) & 7;
+    int a_off[4], b_off[4];
+#pragma unroll
+    for (int sub = 0; sub < 4; ++sub) {
+        const int pc = (sub * 2 + lane / 32) ^ sw;
+        a_off[sub] = (wm * WTM + frow) * DMA64_BK + pc * 8;
+        b_off[sub] = BM * DMA64_BK + ((NB == 1 ? wn * 128 : wn * 64) + frow) * DMA64_BK + pc * 8;
+    }
+    half8_t af[2][FM], bf[2][4];
+    auto one_read = [&](int set, int kt, int sub, int r) {
+        const half_t *st = lds + (kt & 1) * STAGE_HALVES;
+        if (r < FM) af[set][r] = load8(st + a_off[sub] + r * 32 * DMA64_BK);
+        else {
+            const int f = r - FM;
+            const int roff = NB == 1 ? f * 32 : (f / 2) * BN + (f % 2) * 32;
+            bf[set][f] = load8(st + b_off[sub] + roff * DMA64_BK);
+        }
+    };
+
+    float16_t acc[4][FM];
+#pragma unroll
+    for (int f = 0; f < 4; ++f)
+#pragma unroll
+        for (int i = 0; i < FM; ++i)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[f][i][e] = 0.f;
+
+    const int nk = K / DMA64_BK;
+#pragma unroll
+    for (int t = 0; t < LPT; ++t) issue_one(0, t);
+    if (nk > 1) {
+#pragma unroll
+        for (int t = 0; t < LPT / 2; ++t) issue_one(1, t);
+        asm volatile("s_waitcnt vmcnt(8)\n\ts_barrier" ::: "memory");
+    } else {
+        asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+    }
+#pragma unroll
+    for (int r = 0; r < FM + 4; ++r) one_read(0, 0, 0, r);
+
+    constexpr int MM = 4 * FM, RD = FM + 4;
+    // sixteen MFMAs on fragment set `set`; behind MFMA i: one LDS read of the next fragments (i < 8) and, in a
+    // sub-step that issues half a tile, one tile load behind every second MFMA (never two loads back to back:
+    // four waves issuing in step would otherwise fill the address unit's queue and stall on it)
+    auto substep = [&](int set, int next_kt, int next_sub, auto with_issue, int issue_kt, int issue_base) {
+#pragma unroll
+        for (int i = 0; i < MM; ++i) {
+            acc[i / FM][i % FM] =
+                __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[set][i / FM], af[set][i % FM], acc[i / FM][i % FM], 0, 0, 0);
+            if (i < RD) one_read(set ^ 1, next_kt, next_sub, i);
+            if (decltype(with_issue)::value && (i & 1)) issue_one(issue_kt, issue_base + i / 2);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    // Step kt: sub-step 0 issues the second half of tile kt+1, sub-step 3 (behind the barrier that releases
+    // the stage of tile kt) the first half of tile kt+2.
+    int kt = 0;
+    for (; kt + 2 < nk; ++kt) {
+        substep(0, kt, 1, std::true_type{}, kt + 1, LPT / 2);
+        substep(1, kt, 2, std::false_type{}, 0, 0);
+        substep(0, kt, 3, std::false_type{}, 0, 0);
+        // every wave holds the last fragments of this stage; the next tile has landed
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        substep(1, kt + 1, 0, std::true_type{}, kt + 2, 0);
+    }
+    if (kt + 1 < nk) {
+        substep(0, kt, 1, std::true_type{}, kt + 1, LPT / 2);
+        substep(1, kt, 2, std::false_type{}, 0, 0);
+        substep(0, kt, 3, std::false_type{}, 0, 0);
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        substep(1, kt + 1, 0, std::false_type{}, 0, 0);
+        ++kt;
+    }
+    {
+        substep(0, kt, 1, std::false_type{}, 0, 0);
+        substep(1, kt, 2, std::false_type{}, 0, 0);
+        substep(0, kt, 3, std::false_type{}, 0, 0);
+        substep(1, kt, 3, std::false_type{}, 0, 0); // reads a fragment set nobody uses
+    }
+
+    const int mrow = lane % 32, ncol0 = 4 * (lane / 32);
+#pragma unroll
+    for (int i = 0; i < FM; ++i) {
+        const int m = m0 + wm * WTM + i * 32 + mrow;
+        const int mc = m < T ? m : T - 1;
+#pragma unroll
+        for (int j = 0; j < FN; ++j) {
+            const int nb = n0 + (NB == 1 ? wn * 128 : wn * 64) + j * 32 + ncol0;
+            half4_t rv[4];
+            if (NB == 1 && res) {
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    int n = nb + 8 * g;
+                    n = n < N ? n : N - 4;
+                    rv[g] = *reinterpret_cast<const half4_t *>(res + (size_t)mc * ldr + n);
+                }
+            }
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int n = nb + 8 * g;
+                half4_t o;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    if (NB == 2) o[e] = swiglu_to_half(acc[j][i][4 * g + e], acc[2 + j][i][4 * g + e]);
+                    else if (res) o[e] = (half_t)((float)(half_t)acc[j][i][4 * g + e] + (float)rv[g][e]);
+                    else o[e] = (half_t)acc[j][i][4 * g + e];
+                }
+                if (m < T && n < N) *reinterpret_cast<half4_t *>(out + (size_t)m * ldo + n) = o;
+            }
+        }
+    }
+}
+
+template <int NB>
+static int gemm_dma64_launch(const half_t *x, int ldx, const half_t *w, const half_t *w2, const half_t *res, int ldr,
+                             half_t *out, int ldo, int T, int N, int K, hipStream_t s) {
+    constexpr int BM = 256, BN = 256 / NB;
+    const int tiles_m = (T + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
+    const size_t smem = sizeof(half_t) * (size_t)2 * (BM + 256) * DMA64_BK;
+    auto kern = gemm_dma64_kernel<NB>;
+    static std::atomic<uint64_t> attr_done{0};
+    int rc = llm_ensure_max_smem((const void *)kern, smem, attr_done);
+    if (rc != LLM_OK) return rc;
+    kern<<<dim3(tiles_m * tiles_n), dim3(256), smem, s>>>(x, ldx, w, w2, res, ldr, out, ldo, T, N, K, tiles_m, tiles_n);
+    LLM_LAUNCH_CHECK("gemm_dma64_kernel");
+    return LLM_OK;
+}
+
 // out[m][n] = finish(sum over z of ws[z][m][n]) (NB = 2: SiLU(sum of gate slices) * sum of up slices):
 // four columns per thread, slices added in ascending z
 template <int NB>
@@ -974,6 +1172,7 @@ int llm_linear(const uint16_t *x, int ldx, const uint16_t *w, const uint16_t *re
     // 256 x 256 tile as four waves of 128 x 128 (one per SIMD, accumulators in the second register
     // file): a third fewer LDS reads per MFMA than eight waves of 64 x 128, which on this
     // power-limited part is worth 3-12 % with real (non-constant) operands
+    if (K % DMA64_BK == 0) return gemm_dma64_launch<1>(xp, ldx, wp, nullptr, rp, ldr, op, ldo, T, N, K, s);
     return gemm_dma_launch<1, 2, 2, 4, true, 1, 4>(xp, ldx, wp, nullptr, rp, ldr, op, ldo, T, N, K, 1, s);
 }
 
@@ -1009,6 +1208,7 @@ int llm_linear_swiglu(const uint16_t *x, int ldx, const uint16_t *wgate, const u
                                                         pick_splits(2 * (long)((N + 63) / 64), T, N, K, 2), s);
     if ((long)((T + 255) / 256) * ((N + 127) / 128) < 192)
         return gemm_dma_launch<2, 4, 1, 3, false, 2>(xp, ldx, gp, up, nullptr, 0, op, ldo, T, N, K, 1, s);
+    if (K % DMA64_BK == 0) return gemm_dma64_launch<2>(xp, ldx, gp, up, nullptr, 0, op, ldo, T, N, K, s);
     return gemm_dma_launch<2, 2, 2, 4, true, 1, 4>(xp, ldx, gp, up, nullptr, 0, op, ldo, T, N, K, 1, s);
 }
 

@@ -41,9 +41,8 @@ def test_convert_ragged_sizes(gpu, n):
 def test_convert_between_unaligned_buffers(gpu):
     """Source and destination that do not start on a 16-byte boundary take the element-wise kernel."""
     n = 100003
-    src = np.random.default_rng(4).integers(0, 65536, size=n + 8, dtype=np.uint32).astype(np.uint16)
-    d_src, d_dst = gpu.capi.DevBuf.from_host(src), gpu.capi.DevBuf((n + 8,), np.uint16)
-    d_dst.zero()
+    src = np.random.default_rng(4).integers(0, 65536, size=n + 9, dtype=np.uint32).astype(np.uint16)
+    d_src, d_dst = gpu.capi.DevBuf.from_host(src), gpu.capi.DevBuf.from_host(np.zeros(n + 9, np.uint16))
     gpu.capi.check(gpu.lib().llm_bf16_to_fp16(d_src.ptr + 2, d_dst.ptr + 6, n, None))
     out = d_dst.download()
     assert np.array_equal(out[3:3 + n], orc.bf16_to_fp16(src[1:1 + n]))
