@@ -550,8 +550,8 @@ template <int LPT, int MAXT> __device__ __forceinline__ void dma_wait_tiles(int 
 // gate and the same 64 of up), BK = 32, STAGES LDS buffers filled by direct global->LDS loads.
 // Split-K (ws != nullptr): workgroup (tile, z) covers k in [z*kper, (z+1)*kper) and stores its fp32
 // partial tile to ws[z][T][N]; splitk_reduce_kernel sums the slices in ascending z and finishes.
-// PREF: read the next tile's first fragments before the barrier (needs tiles kt and kt+1 landed at
-// barrier kt, so loads run STAGES-2 iterations ahead); otherwise loads run STAGES-1 ahead.
+// Loads run STAGES-1 tiles ahead.  PREF must be false: the pipeline that reads the next tile's first fragments
+// before the barrier is gemm_dma64_kernel's (the 256 x 256 tile of the long prompt passes).
 template <int NB, int WGM, int WGN, int STAGES, bool PREF, int OCC, int FM = 2>
 __global__ __launch_bounds__(WGM * WGN * 64, OCC) void gemm_dma_kernel(const half_t *__restrict__ x, int ldx,
                                                                const half_t *__restrict__ w, const half_t *__restrict__ w2,
@@ -667,76 +667,20 @@ __global__ __launch_bounds__(WGM * WGN * 64, OCC) void gemm_dma_kernel(const hal
 #pragma unroll
     for (int t = 0; t < AHEAD + (PREF ? 1 : 0); ++t)
         if (t < nk) issue(t);
-    // tiles issued so far: min(nk, AHEAD + PREF).  Loop invariant at the top of iteration kt: tiles up to
-    // kt + (PREF ? 1 : 0) have landed for every wave, tiles up to kt + AHEAD - (PREF ? 0 : 1) ... are in flight.
-    if constexpr (PREF) {
-        const int beyond = (nk < AHEAD + 1 ? nk : AHEAD + 1) - 2;
-        if (beyond >= 2) dma_wait_barrier<2 * LPT>();
-        else if (beyond == 1) dma_wait_barrier<LPT>();
-        else dma_wait_barrier<0>();
-        lfrag(0, 0, 0);
-        // One pass = one BK step: 2 x 16 MFMAs on fragment sets 0 and 1.  Set 1 of this step and set 0 of the
-        // next are read from LDS while the MFMAs run (set 0 of a step past the end reads a stale stage and is
-        // never used: no branch inside the pass), the loads of the step AHEAD + 1 further on are issued first.
-        // The instruction order of a pass is written out and pinned (a scheduling fence after every MFMA):
-        // behind MFMA i of the first block one LDS read of set 1, then one tile load; behind MFMA i of the
-        // second block one LDS read of set 0 of the next step.  Left alone the scheduler packs the reads right
-        // in front of their MFMAs to save registers and exposes the LDS latency.
-        constexpr int MM = 4 * FM, RD = FM + 4;
-        static_assert(RD + LPT <= MM, "more loads than MFMAs to hide them behind");
-        auto one_read = [&](int set, int kt, int ks, int r) {
-            const half_t *st = lds + (kt % STAGES) * STAGE_HALVES;
-            if (r < FM) af[set][r] = load8(st + a_off[ks] + r * 32 * DMA_BK);
-            else {
-                const int f = r - FM;
-                const int roff = NB == 1 ? f * 32 : (f / 2) * BN + (f % 2) * 32;
-                bf[set][f] = load8(st + b_off[ks] + roff * DMA_BK);
-            }
-        };
-        auto pass = [&](int kt, auto with_issue) {
-#pragma unroll
-            for (int i = 0; i < MM; ++i) {
-                acc[i / FM][i % FM] =
-                    __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[0][i / FM], af[0][i % FM], acc[i / FM][i % FM], 0, 0, 0);
-                if (i < RD) one_read(1, kt, 1, i);
-                else if (decltype(with_issue)::value && i - RD < LPT) issue_one(kt + AHEAD + 1, i - RD);
-                __builtin_amdgcn_sched_barrier(0);
-            }
-#pragma unroll
-            for (int i = 0; i < MM; ++i) {
-                acc[i / FM][i % FM] =
-                    __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[1][i / FM], af[1][i % FM], acc[i / FM][i % FM], 0, 0, 0);
-                if (i < RD) one_read(0, kt + 1, 0, i);
-                __builtin_amdgcn_sched_barrier(0);
-            }
-        };
-        int kt = 0;
-        for (; kt + AHEAD + 1 < nk; ++kt) {
-            pass(kt, std::true_type{});
-            // tile kt + 2 must have landed; issued after it: tiles kt + 3 .. kt + AHEAD + 1
-            dma_wait_barrier<(AHEAD - 1) * LPT>();
-        }
-        for (; kt < nk; ++kt) {
-            pass(kt, std::false_type{});
-            const int beyond2 = nk - 1 - (kt + 2); // tiles in flight after kt + 2
-            if (AHEAD >= 3 && beyond2 >= 2) dma_wait_barrier<2 * LPT>();
-            else if (beyond2 >= 1) dma_wait_barrier<LPT>();
-            else dma_wait_barrier<0>();
-        }
-    } else {
-        for (int kt = 0; kt < nk; ++kt) {
-            // tile kt landed?  loads issued after it: tiles kt+1 .. min(kt+AHEAD-1, nk-1)
-            const int last = kt + AHEAD - 1 < nk - 1 ? kt + AHEAD - 1 : nk - 1;
-            const int beyond = last - kt;
-            dma_wait_tiles<LPT, AHEAD - 1>(beyond);
-            if (kt + AHEAD < nk) issue(kt + AHEAD);
-            lfrag(0, kt, 0);
-            lfrag(1, kt, 1);
-            __builtin_amdgcn_sched_barrier(0);
-            mma(0);
-            mma(1);
-            __builtin_amdgcn_sched_barrier(0);
-        }
+    // tiles issued so far: min(nk, AHEAD); tiles kt+1 .. kt+AHEAD-1 are in flight at the top of iteration kt
+    static_assert(!PREF, "the read-ahead pipeline lives in gemm_dma64_kernel");
+    for (int kt = 0; kt < nk; ++kt) {
+        // tile kt landed?  loads issued after it: tiles kt+1 .. min(kt+AHEAD-1, nk-1)
+        const int last = kt + AHEAD - 1 < nk - 1 ? kt + AHEAD - 1 : nk - 1;
+        const int beyond = last - kt;
+        dma_wait_tiles<LPT, AHEAD - 1>(beyond);
+        if (kt + AHEAD < nk) issue(kt + AHEAD);
+        lfrag(0, kt, 0);
+        lfrag(1, kt, 1);
+        __builtin_amdgcn_sched_barrier(0);
+        mma(0);
+        mma(1);
+        __builtin_amdgcn_sched_barrier(0);
     }
 
     const int mrow = lane % 32, ncol0 = 4 * (lane / 32);
@@ -1171,9 +1115,9 @@ int llm_linear(const uint16_t *x, int ldx, const uint16_t *w, const uint16_t *re
     }
     // 256 x 256 tile as four waves of 128 x 128 (one per SIMD, accumulators in the second register
     // file): a third fewer LDS reads per MFMA than eight waves of 64 x 128, which on this
-    // power-limited part is worth 3-12 % with real (non-constant) operands
-    if (K % DMA64_BK == 0) return gemm_dma64_launch<1>(xp, ldx, wp, nullptr, rp, ldr, op, ldo, T, N, K, s);
-    return gemm_dma_launch<1, 2, 2, 4, true, 1, 4>(xp, ldx, wp, nullptr, rp, ldr, op, ldo, T, N, K, 1, s);
+    // power-limited part is worth 3-12 % with real (non-constant) operands; BK = 64 so that tile loads
+    // fetch whole cache lines
+    return gemm_dma64_launch<1>(xp, ldx, wp, nullptr, rp, ldr, op, ldo, T, N, K, s); // K % 64 == 0 was checked
 }
 
 int llm_linear_swiglu(const uint16_t *x, int ldx, const uint16_t *wgate, const uint16_t *wup, uint16_t *out,
@@ -1208,8 +1152,7 @@ int llm_linear_swiglu(const uint16_t *x, int ldx, const uint16_t *wgate, const u
                                                         pick_splits(2 * (long)((N + 63) / 64), T, N, K, 2), s);
     if ((long)((T + 255) / 256) * ((N + 127) / 128) < 192)
         return gemm_dma_launch<2, 4, 1, 3, false, 2>(xp, ldx, gp, up, nullptr, 0, op, ldo, T, N, K, 1, s);
-    if (K % DMA64_BK == 0) return gemm_dma64_launch<2>(xp, ldx, gp, up, nullptr, 0, op, ldo, T, N, K, s);
-    return gemm_dma_launch<2, 2, 2, 4, true, 1, 4>(xp, ldx, gp, up, nullptr, 0, op, ldo, T, N, K, 1, s);
+    return gemm_dma64_launch<2>(xp, ldx, gp, up, nullptr, 0, op, ldo, T, N, K, s);
 }
 
 int llm_norm_linear(const uint16_t *x, const uint16_t *gain, double eps, const uint16_t *w, uint16_t *out, int N, int K,
