@@ -284,7 +284,8 @@ def power_ceiling(pkg, a):
     with SmiSampler() as smi:
         time.sleep(1.0)
         res["idle"] = smi.window(time.time() - 1.0, time.time())
-        for kind, name in ((0, "mfma_only_constant_operands"), (1, "mfma_only_random_operands")):
+        for kind, name in ((0, "mfma_only_constant_operands"), (1, "mfma_only_random_operands"),
+                           (2, "mfma_16x16x32_only_constant_operands"), (3, "mfma_16x16x32_only_random_operands")):
             tf, ms = C.c_double(0), C.c_float(0)
             t0 = time.time()
             pkg.capi.check(lib.llm_mfma_probe(kind, C.c_float(2500.0), C.byref(tf), C.byref(ms), None))

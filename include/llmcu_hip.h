@@ -242,10 +242,11 @@ int llm_sample_candidates(const uint16_t *logits_dev, const float *exp_table_dev
                           void *out_dev, llm_stream_t stream);
 
 /* ---- measurement aid ---------------------------------------------------------------------------- */
-/* No counterpart in the reference.  Runs nothing but v_mfma_f32_32x32x16_f16 on every CU for about
- * ms_target milliseconds and reports the sustained rate: kind 0 with constant operands, kind 1 with
- * operands distributed like the prompt pass's (N(0,1) activations, N(0,0.02) weights).  The second is
- * the ceiling that the power limit of the board leaves to the prompt-pass GEMMs. */
+/* No counterpart in the reference.  Runs nothing but MFMAs on every CU for about ms_target milliseconds
+ * and reports the sustained rate: kind 0 with constant operands, kind 1 with operands distributed like
+ * the prompt pass's (N(0,1) activations, N(0,0.02) weights), both with v_mfma_f32_32x32x16_f16; kinds 2
+ * and 3 the same with v_mfma_f32_16x16x32_f16.  The random-operand figures are the ceiling that the
+ * power limit of the board leaves to the prompt-pass GEMMs. */
 int llm_mfma_probe(int kind, float ms_target, double *tflops, float *ms_out, llm_stream_t stream);
 
 /* ---- one decode token in one launch ------------------------------------------------------------- */

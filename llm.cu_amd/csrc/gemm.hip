@@ -736,21 +736,20 @@ __global__ __launch_bounds__(WGM * WGN * 64, OCC) void gemm_dma_kernel(const hal
     }
 }
 
-// The 256 x 256 tile of gemm_dma_kernel<NB,2,2,4,true,1,4> with BK = 64: a tile row is 128 bytes, so every
-// lane group of a tile load fetches a whole cache line (8 rows x 128 B per wave instruction instead of 16 rows
-// x 64 B), and there is one workgroup barrier per 64 k instead of per 32.  Two LDS stages of 64 KB.  A step is
-// four sub-steps of 16 MFMAs on alternating fragment sets; the fragments of a sub-step are read during the one
-// before it.  The barrier sits between sub-steps 2 and 3: by then every wave has read the last fragments of
-// the current stage, and the next tile (issued during sub-step 3 of the previous step) must have landed; in
-// sub-step 3 the first fragments of the next tile are read and the loads of the tile after it are issued
-// into the stage that has just been released.
 #define DMA64_BK 64
+// 256 x 256 tile, BK = 64, four waves of 128 x 128, on v_mfma_f32_16x16x32_f16 (64 accumulators of 4 registers
+// per wave).  With operands that toggle like activations and weights this instruction sustains about 13 % more
+// flops under the board's power limit than v_mfma_f32_32x32x16_f16 (it moves a fifth fewer register bytes per
+// flop: the accumulator traffic halves).  A step is two sub-steps of 64 MFMAs on alternating fragment sets (8
+// activation and 8 weight fragments each, read during the sub-step before); the workgroup barrier sits between
+// the two: by then every wave has read the last fragments of the current stage and the next tile (issued
+// during the previous step's second sub-step, one load behind every fourth MFMA) must have landed.
 template <int NB>
 __global__ __launch_bounds__(256, 1) void gemm_dma64_kernel(const half_t *__restrict__ x, int ldx, const half_t *__restrict__ w,
-                                                            const half_t *__restrict__ w2, const half_t *res, int ldr,
-                                                            half_t *out, int ldo, int T, int N, int K, int tiles_m,
-                                                            int tiles_n) {
-    constexpr int FM = 4, WTM = 128, BM = 256, BROWS = 256, BN = BROWS / NB, FN = 4 / NB;
+                                                           const half_t *__restrict__ w2, const half_t *res, int ldr,
+                                                           half_t *out, int ldo, int T, int N, int K, int tiles_m,
+                                                           int tiles_n) {
+    constexpr int WTM = 128, BM = 256, BROWS = 256, BN = BROWS / NB;
     constexpr int STAGE_HALVES = (BM + BROWS) * DMA64_BK;
     constexpr int LPT = (BM + BROWS) / 8 / 4; // 16 load instructions per wave per tile
     constexpr int TA = BM / 8 / 4, TB1 = BN / 8 / 4;
@@ -774,8 +773,6 @@ __global__ __launch_bounds__(256, 1) void gemm_dma64_kernel(const half_t *__rest
     const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid / 64), lane = tid % 64;
     const int wm = wave % 2, wn = wave / 2;
 
-    // loader: instruction q = wave + 4 t moves stage rows 8q .. 8q+7 (q < 32: A rows, else B rows), 128 B each;
-    // lane -> row lane/8, LDS chunk lane%8, which holds global chunk (lane%8) ^ ((row>>1)&7)
     const __amdgpu_buffer_rsrc_t rs_x =
         __builtin_amdgcn_make_buffer_rsrc((void *)x, 0, ((T - 1) * ldx + K) * (int)sizeof(half_t), 0x00020000);
     const __amdgpu_buffer_rsrc_t rs_w = __builtin_amdgcn_make_buffer_rsrc((void *)w, 0, N * K * (int)sizeof(half_t), 0x00020000);
@@ -806,122 +803,109 @@ __global__ __launch_bounds__(256, 1) void gemm_dma64_kernel(const half_t *__rest
         else __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_w2, dst, 16, goff[t], k0, 0, 0);
     };
 
-    const int frow = lane % 32, sw = (frow >> 1) & 7;
-    int a_off[4], b_off[4];
+    // fragment of a 16-row block for k-step ks (32 k): lane -> row lane%16, 16-byte chunk 4 ks + lane/16
+    const int frow = lane % 16, sw = frow >> 1;
+    int a_off[2], b_off[2];
 #pragma unroll
-    for (int sub = 0; sub < 4; ++sub) {
-        const int pc = (sub * 2 + lane / 32) ^ sw;
-        a_off[sub] = (wm * WTM + frow) * DMA64_BK + pc * 8;
-        b_off[sub] = BM * DMA64_BK + ((NB == 1 ? wn * 128 : wn * 64) + frow) * DMA64_BK + pc * 8;
+    for (int ks = 0; ks < 2; ++ks) {
+        const int pc = (ks * 4 + lane / 16) ^ sw;
+        a_off[ks] = (wm * WTM + frow) * DMA64_BK + pc * 8;
+        b_off[ks] = BM * DMA64_BK + ((NB == 1 ? wn * 128 : wn * 64) + frow) * DMA64_BK + pc * 8;
     }
-    half8_t af[2][FM], bf[2][4];
-    auto one_read = [&](int set, int kt, int sub, int r) {
+    half8_t af[2][8], bf[2][8];
+    auto one_read = [&](int set, int kt, int ks, int r) {
         const half_t *st = lds + (kt & 1) * STAGE_HALVES;
-        if (r < FM) af[set][r] = load8(st + a_off[sub] + r * 32 * DMA64_BK);
+        if (r < 8) af[set][r] = load8(st + a_off[ks] + r * 16 * DMA64_BK);
         else {
-            const int f = r - FM;
-            const int roff = NB == 1 ? f * 32 : (f / 2) * BN + (f % 2) * 32;
-            bf[set][f] = load8(st + b_off[sub] + roff * DMA64_BK);
+            const int f = r - 8;
+            const int roff = NB == 1 ? f * 16 : (f / 4) * BN + (f % 4) * 16;
+            bf[set][f] = load8(st + b_off[ks] + roff * DMA64_BK);
         }
     };
 
-    float16_t acc[4][FM];
+    float4_t acc[8][8]; // [weight block][activation block]
 #pragma unroll
-    for (int f = 0; f < 4; ++f)
+    for (int f = 0; f < 8; ++f)
 #pragma unroll
-        for (int i = 0; i < FM; ++i)
+        for (int i = 0; i < 8; ++i)
 #pragma unroll
-            for (int e = 0; e < 16; ++e) acc[f][i][e] = 0.f;
+            for (int e = 0; e < 4; ++e) acc[f][i][e] = 0.f;
 
     const int nk = K / DMA64_BK;
 #pragma unroll
     for (int t = 0; t < LPT; ++t) issue_one(0, t);
     if (nk > 1) {
 #pragma unroll
-        for (int t = 0; t < LPT / 2; ++t) issue_one(1, t);
-        asm volatile("s_waitcnt vmcnt(8)\n\ts_barrier" ::: "memory");
+        for (int t = 0; t < LPT; ++t) issue_one(1, t);
+        asm volatile("s_waitcnt vmcnt(16)\n\ts_barrier" ::: "memory");
     } else {
         asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
     }
 #pragma unroll
-    for (int r = 0; r < FM + 4; ++r) one_read(0, 0, 0, r);
+    for (int r = 0; r < 16; ++r) one_read(0, 0, 0, r);
 
-    constexpr int MM = 4 * FM, RD = FM + 4;
-    // sixteen MFMAs on fragment set `set`; behind MFMA i: one LDS read of the next fragments (i < 8) and, in a
-    // sub-step that issues half a tile, one tile load behind every second MFMA (never two loads back to back:
-    // four waves issuing in step would otherwise fill the address unit's queue and stall on it)
-    auto substep = [&](int set, int next_kt, int next_sub, auto with_issue, int issue_kt, int issue_base) {
+    // 64 MFMAs on fragment set `set`; behind MFMA i: one LDS read of the next fragments (every second MFMA, 16 in
+    // all, weight fragment 0 and the activation fragments first: the order of use) and, in a sub-step that issues
+    // a tile, one tile load behind every fourth MFMA
+    auto substep = [&](int set, int next_kt, int next_ks, auto with_issue, int issue_kt) {
 #pragma unroll
-        for (int i = 0; i < MM; ++i) {
-            acc[i / FM][i % FM] =
-                __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[set][i / FM], af[set][i % FM], acc[i / FM][i % FM], 0, 0, 0);
-            if (i < RD) one_read(set ^ 1, next_kt, next_sub, i);
-            if (decltype(with_issue)::value && (i & 1)) issue_one(issue_kt, issue_base + i / 2);
+        for (int i = 0; i < 64; ++i) {
+            const int f = i / 8, m = i % 8;
+            // as text, accumulator tied to itself: with the builtin the register allocator moves the 64
+            // accumulators between the two register files around the MFMAs (hundreds of copies per step)
+            asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc[f][m]) : "v"(bf[set][f]), "v"(af[set][m]));
+            if ((i & 1) == 0) {
+                const int r = i / 2; // 0..31: 16 reads in the first half of the sub-step
+                if (r < 16) one_read(set ^ 1, next_kt, next_ks, r == 0 ? 8 : (r <= 8 ? r - 1 : r));
+            }
+            if (decltype(with_issue)::value && (i & 3) == 3) issue_one(issue_kt, i / 4);
             __builtin_amdgcn_sched_barrier(0);
         }
     };
-    // Step kt: sub-step 0 issues the second half of tile kt+1, sub-step 3 (behind the barrier that releases
-    // the stage of tile kt) the first half of tile kt+2.
     int kt = 0;
     for (; kt + 2 < nk; ++kt) {
-        substep(0, kt, 1, std::true_type{}, kt + 1, LPT / 2);
-        substep(1, kt, 2, std::false_type{}, 0, 0);
-        substep(0, kt, 3, std::false_type{}, 0, 0);
+        substep(0, kt, 1, std::false_type{}, 0);
         // every wave holds the last fragments of this stage; the next tile has landed
         asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
-        substep(1, kt + 1, 0, std::true_type{}, kt + 2, 0);
+        substep(1, kt + 1, 0, std::true_type{}, kt + 2);
     }
-    if (kt + 1 < nk) {
-        substep(0, kt, 1, std::true_type{}, kt + 1, LPT / 2);
-        substep(1, kt, 2, std::false_type{}, 0, 0);
-        substep(0, kt, 3, std::false_type{}, 0, 0);
+    for (; kt < nk; ++kt) {
+        substep(0, kt, 1, std::false_type{}, 0);
         asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
-        substep(1, kt + 1, 0, std::false_type{}, 0, 0);
-        ++kt;
+        substep(1, kt + 1, 0, std::false_type{}, 0); // past the last tile: reads a stage nobody uses
     }
-    {
-        substep(0, kt, 1, std::false_type{}, 0, 0);
-        substep(1, kt, 2, std::false_type{}, 0, 0);
-        substep(0, kt, 3, std::false_type{}, 0, 0);
-        substep(1, kt, 3, std::false_type{}, 0, 0); // reads a fragment set nobody uses
-    }
+    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory"); // the compiler does not see the MFMAs' result latency
 
-    const int mrow = lane % 32, ncol0 = 4 * (lane / 32);
+    // lane l of a 16 x 16 block holds activation row l%16 and weight rows 4 (l/16) .. + 3: four output columns
+    const int mrow = lane % 16, ncol0 = 4 * (lane / 16);
 #pragma unroll
-    for (int i = 0; i < FM; ++i) {
-        const int m = m0 + wm * WTM + i * 32 + mrow;
+    for (int i = 0; i < 8; ++i) {
+        const int m = m0 + wm * WTM + i * 16 + mrow;
         const int mc = m < T ? m : T - 1;
 #pragma unroll
-        for (int j = 0; j < FN; ++j) {
-            const int nb = n0 + (NB == 1 ? wn * 128 : wn * 64) + j * 32 + ncol0;
-            half4_t rv[4];
+        for (int j = 0; j < 8 / NB; ++j) {
+            const int n = n0 + (NB == 1 ? wn * 128 : wn * 64) + j * 16 + ncol0;
+            half4_t o;
             if (NB == 1 && res) {
+                const int nc = n < N ? n : N - 4;
+                const half4_t rv = *reinterpret_cast<const half4_t *>(res + (size_t)mc * ldr + nc);
 #pragma unroll
-                for (int g = 0; g < 4; ++g) {
-                    int n = nb + 8 * g;
-                    n = n < N ? n : N - 4;
-                    rv[g] = *reinterpret_cast<const half4_t *>(res + (size_t)mc * ldr + n);
-                }
-            }
-#pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                const int n = nb + 8 * g;
-                half4_t o;
+                for (int e = 0; e < 4; ++e) o[e] = (half_t)((float)(half_t)acc[j][i][e] + (float)rv[e]);
+            } else {
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
-                    if (NB == 2) o[e] = swiglu_to_half(acc[j][i][4 * g + e], acc[2 + j][i][4 * g + e]);
-                    else if (res) o[e] = (half_t)((float)(half_t)acc[j][i][4 * g + e] + (float)rv[g][e]);
-                    else o[e] = (half_t)acc[j][i][4 * g + e];
+                    if (NB == 2) o[e] = swiglu_to_half(acc[j][i][e], acc[4 + j][i][e]);
+                    else o[e] = (half_t)acc[j][i][e];
                 }
-                if (m < T && n < N) *reinterpret_cast<half4_t *>(out + (size_t)m * ldo + n) = o;
             }
+            if (m < T && n < N) *reinterpret_cast<half4_t *>(out + (size_t)m * ldo + n) = o;
         }
     }
 }
 
 template <int NB>
 static int gemm_dma64_launch(const half_t *x, int ldx, const half_t *w, const half_t *w2, const half_t *res, int ldr,
-                             half_t *out, int ldo, int T, int N, int K, hipStream_t s) {
+                            half_t *out, int ldo, int T, int N, int K, hipStream_t s) {
     constexpr int BM = 256, BN = 256 / NB;
     const int tiles_m = (T + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
     const size_t smem = sizeof(half_t) * (size_t)2 * (BM + 256) * DMA64_BK;

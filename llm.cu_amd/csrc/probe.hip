@@ -6,19 +6,19 @@
 
 #include "common.hpp"
 
-// Every wavefront: `iters` rounds of sixteen v_mfma_f32_32x32x16_f16 over four A and four B operand sets (every
-// MFMA sees operands that differ from its predecessor's, as in a GEMM) into eight accumulators (128 accumulator
-// registers, no dependency stalls).  kind 0: all operands 1.0; kind 1: normal(0, 1) activations against
-// normal(0, 0.02) weights from a counter-based generator, different in every lane and set.
-__global__ __launch_bounds__(256) void mfma_probe_kernel(float *sink, int iters, int kind) {
+// Every wavefront: `iters` rounds of MFMAs over four A and four B operand sets (every MFMA sees operands that
+// differ from its predecessor's, as in a GEMM) into 128 accumulator registers (no dependency stalls): sixteen
+// v_mfma_f32_32x32x16_f16 into eight accumulators, or (SMALL) thirty-two v_mfma_f32_16x16x32_f16 into
+// thirty-two -- the same flops per round.  kind bit 0 clear: all operands 1.0; set: normal(0, 1) activations
+// against normal(0, 0.02) weights from a counter-based generator, different in every lane and set.
+template <bool SMALL> __global__ __launch_bounds__(256) void mfma_probe_kernel(float *sink, int iters, int kind) {
     half8_t a[4], b[4];
-    float16_t acc[8];
     const unsigned id = blockIdx.x * blockDim.x + threadIdx.x;
 #pragma unroll
     for (int p = 0; p < 4; ++p) {
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-            if (kind == 0) {
+            if ((kind & 1) == 0) {
                 a[p][i] = (half_t)1.0f;
                 b[p][i] = (half_t)1.0f;
             } else {
@@ -33,29 +33,50 @@ __global__ __launch_bounds__(256) void mfma_probe_kernel(float *sink, int iters,
             }
         }
     }
-#pragma unroll
-    for (int j = 0; j < 8; ++j)
-#pragma unroll
-        for (int e = 0; e < 16; ++e) acc[j][e] = 0.f;
-    for (int it = 0; it < iters; ++it) {
-#pragma unroll
-        for (int j = 0; j < 16; ++j)
-            acc[j & 7] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[j & 3], b[(j >> 2) & 3], acc[j & 7], 0, 0, 0);
-    }
     float s = 0.f;
+    if constexpr (SMALL) {
+        float4_t acc[32];
 #pragma unroll
-    for (int j = 0; j < 8; ++j)
+        for (int j = 0; j < 32; ++j)
 #pragma unroll
-        for (int e = 0; e < 16; ++e) s += acc[j][e];
+            for (int e = 0; e < 4; ++e) acc[j][e] = 0.f;
+        for (int it = 0; it < iters; ++it) {
+#pragma unroll
+            for (int j = 0; j < 32; ++j)
+                // written as text so that every accumulator stays in place (the builtin form made the register
+                // allocator copy half of them through a scratch tuple around each MFMA)
+                asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc[j]) : "v"(a[j & 3]), "v"(b[(j >> 2) & 3]));
+        }
+#pragma unroll
+        for (int j = 0; j < 32; ++j)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) s += acc[j][e];
+    } else {
+        float16_t acc[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[j][e] = 0.f;
+        for (int it = 0; it < iters; ++it) {
+#pragma unroll
+            for (int j = 0; j < 16; ++j)
+                acc[j & 7] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[j & 3], b[(j >> 2) & 3], acc[j & 7], 0, 0, 0);
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) s += acc[j][e];
+    }
     if (s == 123.456f) sink[0] = s; // keeps the loop alive
 }
 
 extern "C" {
 
 // Runs the probe for about `ms_target` milliseconds on `stream` and returns the sustained rate.
-// kind: 0 constant operands, 1 random operands shaped like the prompt pass's (N(0,1) x N(0,0.02)).
+// kind: 0 constant operands, 1 random operands shaped like the prompt pass's (N(0,1) x N(0,0.02)), both with
+// v_mfma_f32_32x32x16_f16; 2 and 3: the same with v_mfma_f32_16x16x32_f16.
 int llm_mfma_probe(int kind, float ms_target, double *tflops, float *ms_out, llm_stream_t stream) {
-    LLM_REQUIRE(tflops && (kind == 0 || kind == 1) && ms_target > 0.f, "llm_mfma_probe: arguments");
+    LLM_REQUIRE(tflops && kind >= 0 && kind <= 3 && ms_target > 0.f, "llm_mfma_probe: arguments");
     int cus = 0;
     int rc = llm_cu_count_cached(&cus);
     if (rc != LLM_OK) return rc;
@@ -68,7 +89,8 @@ int llm_mfma_probe(int kind, float ms_target, double *tflops, float *ms_out, llm
     const int grid = cus * 2; // 8 wavefronts per CU, two per SIMD
     auto run = [&](int iters, float *ms) -> int {
         LLM_HIP_CHECK(hipEventRecord(e0, s));
-        mfma_probe_kernel<<<dim3(grid), dim3(256), 0, s>>>(sink, iters, kind);
+        if (kind & 2) mfma_probe_kernel<true><<<dim3(grid), dim3(256), 0, s>>>(sink, iters, kind);
+        else mfma_probe_kernel<false><<<dim3(grid), dim3(256), 0, s>>>(sink, iters, kind);
         LLM_LAUNCH_CHECK("mfma_probe_kernel");
         LLM_HIP_CHECK(hipEventRecord(e1, s));
         LLM_HIP_CHECK(hipEventSynchronize(e1));
