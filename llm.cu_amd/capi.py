@@ -11,7 +11,8 @@ import os
 import numpy as np
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(HERE, "libllmcu.so")
+# LLMCU_LIB names another build of the same library (kernel experiments side by side with the shipped build)
+LIB_PATH = os.environ.get("LLMCU_LIB") or os.path.join(HERE, "libllmcu.so")
 
 LLM_OK, LLM_ERR_INVALID, LLM_ERR_HIP, LLM_ERR_NO_DEVICE = 0, 1, 2, 3
 

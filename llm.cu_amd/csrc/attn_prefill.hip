@@ -1,6 +1,11 @@
 // Causal GQA attention for a block of query rows (prompt pass): streaming
-// softmax over 64-key tiles on v_mfma_f32_32x32x16_f16; the [H,T,T] score
+// softmax over key tiles on v_mfma_f32_32x32x16_f16; the [H,T,T] score
 // tensor of the reference (src/inference/inference.cu:698-947) never exists.
+//
+// Two kernels share the arithmetic.  attn_prefill_kernel (any supported head
+// size and group) is described next; attn_prefill_pipe_kernel (head size 128,
+// four query heads per KV head, the LLaMA3-8B shape) is the software-pipelined
+// form further down.
 //
 // One workgroup = one KV head x 64 query rows (two 32-row tiles); each
 // wavefront serves one query head on one tile, so the G heads of a group and
@@ -30,6 +35,9 @@
 
 #define AP_BQ 32
 #define AP_BKEY 64
+#ifndef AP_PIPE_MIN_ROWS
+#define AP_PIPE_MIN_ROWS 64 // shorter blocks of rows take attn_prefill_kernel
+#endif
 
 // Workgroup = one KV head x AP_QT query tiles (2, or 1 for groups of 8 heads); wavefront w serves query head
 // kvh*G + w%G on tile w/G, so G*AP_QT wavefronts share every K/V tile.  K/V
@@ -334,6 +342,287 @@ __global__ __launch_bounds__(G *AP_QT * 64) void attn_prefill_kernel(const half_
     }
 }
 
+#define AP_LDS_PTR(p) ((__attribute__((address_space(3))) void *)(p))
+
+// ---- software-pipelined form for head size 128 and four query heads per KV head -----------------------------
+//
+// Same workgroup shape (one KV head x 64 query rows, wavefront = one head x 32 rows, two wavefronts per SIMD) and
+// the same two transposed products, organised around what bounds the kernel on this part: board power.  Time
+// follows the energy of the instructions issued, so the kernel issues fewer of them:
+//  * The unit of work is a chunk of 32 keys.  One iteration computes the scores of chunk c + 1 (8 MFMAs), the
+//    probabilities of chunk c (16 values per lane) and O^T += V^T . P^T of chunk c - 1 (8 MFMAs); the softmax
+//    instructions sit between the MFMAs (a SIMD takes about four vector instructions under each MFMA), two
+//    score and two probability sets alternate, and two iterations form one trip of the loop.
+//  * K and V^T tiles of 64 keys travel from global memory straight into a ring of four LDS stages
+//    (buffer_load ... lds, no staging registers, no LDS stores); a lane fetches the 16-byte chunk that the
+//    bank swizzle assigns to its LDS slot.  One workgroup barrier per tile.
+//  * The softmax keeps a reference maximum per query that moves only when a probability would leave the fp16
+//    range (then the row sum reads infinite): the running maximum is not computed per chunk, and O^T is
+//    rescaled a handful of times per query instead of whenever any lane's maximum moves.  Probabilities are
+//    2^(s c - m_ref) <= 65504 in fp16, sums and O^T in fp32, so the result is the same softmax: O^T / l.
+typedef uint32_t ap_u4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t ap_u8_t __attribute__((ext_vector_type(8)));
+
+template <int G>
+__global__ __launch_bounds__(G * 128, 1) void attn_prefill_pipe_kernel(const half_t *__restrict__ q, int ldq,
+                                                                       const half_t *__restrict__ kc,
+                                                                       const half_t *__restrict__ vc,
+                                                                       half_t *__restrict__ out, int ldo, int T,
+                                                                       int pos0, int max_pos) {
+    static_assert(G == 4, "eight wavefronts, two per SIMD");
+    constexpr int HD = 128, NW = 2 * G, THREADS = NW * 64;
+    constexpr int LPT = 32 / NW;            // tile-load instructions per wavefront and tile
+    constexpr int HALF_TILE = 32 * HD;      // halves of a 32-key K half-tile (8 KB)
+    constexpr int TILE = 2 * HALF_TILE;     // 64 keys x 128 dims, K or V^T (16 KB)
+    constexpr int VRING = 4 * TILE;         // V ring behind the K ring
+    extern __shared__ __attribute__((aligned(16))) half_t smem[];
+
+    const int blk = gridDim.y - 1 - blockIdx.y; // longest rows first
+    const int kvh = blockIdx.x;
+    const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid / 64), lane = tid % 64;
+    const int head = kvh * G + wave % G;
+    const int n = lane % 32, hb = lane / 32;
+    const int q0 = blk * 64;          // first row of the workgroup
+    const int q0w = q0 + 32 * (wave / G); // first row of this wavefront
+    int q_last = q0 + 63;
+    if (q_last > T - 1) q_last = T - 1;
+    const int nc = (pos0 + q_last) / 32 + 1; // 32-key chunks the workgroup visits
+    const int n_tiles = (nc + 1) / 2;
+    const int n_plain = (pos0 + q0w + 1) / 32; // chunks that no query of the wavefront has masked keys in
+
+    const int r = q0w + n;
+    const int qrow = r < T ? r : T - 1;
+    const int qpos = pos0 + r;
+    half8_t qf[8];
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) qf[ks] = load8(q + (size_t)qrow * ldq + (size_t)head * HD + 16 * ks + 8 * hb);
+
+    // tile loads straight into LDS: wave instruction i' = wave + NW t covers 1 KB = 4 K rows or 8 V^T rows; lane l
+    // writes 16 bytes at 16 l and fetches the 16-byte chunk of its row that the swizzle puts there
+    const __amdgpu_buffer_rsrc_t rs_k = __builtin_amdgcn_make_buffer_rsrc((void *)(kc + (size_t)kvh * max_pos * HD), 0,
+                                                                          max_pos * HD * 2, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rs_v = __builtin_amdgcn_make_buffer_rsrc((void *)(vc + (size_t)kvh * HD * max_pos), 0,
+                                                                          HD * max_pos * 2, 0x00020000);
+    const int krow_l = 4 * wave + lane / 16;
+    const uint32_t kvoff = (uint32_t)krow_l * 256u + (uint32_t)(((lane % 16) ^ (krow_l & 15)) * 16);
+    const int vrow_l = 8 * wave + lane / 8;
+    const uint32_t vvoff = (uint32_t)vrow_l * (uint32_t)max_pos * 2u + (uint32_t)(((lane % 8) ^ ((vrow_l >> 1) & 7)) * 16);
+    auto issue = [&](int tile, int t) __attribute__((always_inline)) { // t < LPT: first half K, second half V
+        const int st = tile & 3;
+        if (t < LPT / 2) {
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_k, AP_LDS_PTR(smem + st * TILE + (wave + NW * t) * 512), 16, kvoff,
+                                                     (uint32_t)tile * 64u * 256u + (uint32_t)t * (4u * NW * 256u), 0, 0);
+        } else {
+            const int tt = t - LPT / 2;
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_v, AP_LDS_PTR(smem + VRING + st * TILE + (wave + NW * tt) * 512), 16,
+                                                     vvoff, (uint32_t)tile * 128u + (uint32_t)tt * (16u * NW) * (uint32_t)max_pos,
+                                                     0, 0);
+        }
+    };
+    auto clamp_tile = [&](int tile) __attribute__((always_inline)) { return tile < n_tiles ? tile : n_tiles - 1; };
+
+    // fragment addresses (halves): K rows in the order pi(m) (bits 2 and 3 swapped), 16-byte chunks swizzled
+    const int pm = (n & ~0xC) | ((n & 8) >> 1) | ((n & 4) << 1);
+    int klane[8], vlane[2][2];
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) klane[ks] = pm * 128 + (((2 * ks + hb) ^ (pm & 15)) * 8);
+#pragma unroll
+    for (int cp = 0; cp < 2; ++cp)
+#pragma unroll
+        for (int u = 0; u < 2; ++u) vlane[cp][u] = VRING + n * 64 + (((4 * cp + 2 * u + hb) ^ ((n >> 1) & 7)) * 8);
+
+    float16_t S[2];
+    ap_u8_t P[2];
+    float16_t O[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) O[t][e] = 0.f;
+#pragma unroll
+    for (int b = 0; b < 2; ++b) {
+#pragma unroll
+        for (int e = 0; e < 16; ++e) S[b][e] = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) P[b][e] = 0u;
+    }
+    float m_used = -FLT_MAX, l_run = 0.f, sum = 0.f;
+    const float c2 = 1.44269504088896341f / sqrtf((float)HD);
+
+    auto xhalf = [&](float x, float &lo, float &hi) __attribute__((always_inline)) {
+        auto rr = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+        lo = __uint_as_float(rr[0]);
+        hi = __uint_as_float(rr[1]);
+    };
+    // probabilities of elements 2g, 2g+1 against the reference maximum in use
+    auto slice = [&](float16_t &s, ap_u8_t &p, int g) __attribute__((always_inline)) {
+        const float nm = -m_used;
+        const float p0 = __builtin_amdgcn_exp2f(fmaf(s[2 * g], c2, nm));
+        const float p1 = __builtin_amdgcn_exp2f(fmaf(s[2 * g + 1], c2, nm));
+        const half2_t h = {(half_t)p0, (half_t)p1};
+        p[g] = __builtin_bit_cast(uint32_t, h);
+        sum = __builtin_amdgcn_fdot2(h, half2_t{(half_t)1.0f, (half_t)1.0f}, sum, false);
+    };
+    // The reference maximum only moves when a probability would leave the fp16 range (the row sum turns
+    // infinite): then the true running maximum becomes the reference, O^T and the row sum are rescaled and
+    // the chunk's probabilities are computed again.  The first chunk always comes through here.
+    auto settle = [&](float16_t &s, ap_u8_t &p) __attribute__((always_inline)) {
+        const bool bad = !(sum < 3.0e38f);
+        if (__builtin_amdgcn_ballot_w64(bad) != 0) {
+            asm volatile("s_nop 15\n\ts_nop 15" ::: "memory"); // MFMAs written as text: their result latency is not tracked
+            float mx = -FLT_MAX;
+#pragma unroll
+            for (int e = 0; e < 16; ++e) mx = fmaxf(mx, s[e]);
+            float lo, hi;
+            xhalf(mx, lo, hi);
+            const float m_new = fmaxf(m_used, fmaxf(lo, hi) * c2);
+            const float alpha = __builtin_amdgcn_exp2f(m_used - m_new);
+            l_run *= alpha;
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) O[t][e] *= alpha;
+            m_used = m_new;
+            sum = 0.f;
+#pragma unroll
+            for (int g = 0; g < 8; ++g) slice(s, p, g);
+        }
+        l_run += sum;
+    };
+    // causal mask of chunk c on the scores in s: accumulator e is key 32 c + 16 (e / 8) + 8 hb + e % 8
+    auto mask = [&](float16_t &s, int c) __attribute__((always_inline)) {
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            const int key = 32 * c + 16 * (e / 8) + 8 * hb + (e % 8);
+            s[e] = key <= qpos ? s[e] : -FLT_MAX;
+        }
+    };
+    auto pfrag = [&](ap_u8_t &p, int u) __attribute__((always_inline)) {
+        ap_u4_t rr = u == 0 ? __builtin_shufflevector(p, p, 0, 1, 2, 3) : __builtin_shufflevector(p, p, 4, 5, 6, 7);
+        return __builtin_bit_cast(half8_t, rr);
+    };
+
+    // One pipelined iteration on chunk c (PAR = c % 2): scores of chunk c + 1 into s_nxt, probabilities of chunk c
+    // from s_cur into p_cur, O^T += V^T(chunk c - 1) . p_prv.  Every iteration does all three: past the last
+    // chunk the scores are computed from a stale ring slot and never used, and in front of the first chunk the
+    // probabilities are zero and the V region was cleared.
+    auto step = [&](float16_t &s_cur, float16_t &s_nxt, ap_u8_t &p_cur, ap_u8_t &p_prv, int c, auto par_c,
+                    int dma_tile) __attribute__((always_inline)) {
+        constexpr int PAR = decltype(par_c)::value;
+        const int koff = ((c + 1) & 7) * HALF_TILE;
+        const int voff = (((c - 1) >> 1) & 3) * TILE;
+        constexpr int RA = 3; // fragments read ahead
+        half8_t kf[RA], vf[RA];
+        auto rd = [&](int grp) __attribute__((always_inline)) {
+            kf[grp % RA] = load8(smem + koff + klane[grp]);
+            vf[grp % RA] = load8(smem + voff + vlane[1 - PAR][grp / 4] + (grp % 4) * 2048);
+        };
+#pragma unroll
+        for (int g0 = 0; g0 < RA - 1; ++g0) rd(g0);
+        if (c >= n_plain) {
+            asm volatile("s_nop 15\n\ts_nop 15" ::: "memory"); // the scores come from MFMAs written as text
+            mask(s_cur, c);
+        }
+        sum = 0.f;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const int grp = i / 2;
+            if (i % 2 == 0 && grp + RA - 1 < 8) rd(grp + RA - 1);
+            if (i % 2 == 0) {
+                if (grp == 0) asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(s_nxt) : "v"(kf[grp % RA]), "v"(qf[grp]));
+                else asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(s_nxt) : "v"(kf[grp % RA]), "v"(qf[grp]));
+            } else {
+                const int t = grp % 4, u = grp / 4;
+                asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(O[t]) : "v"(vf[grp % RA]), "v"(pfrag(p_prv, u)));
+            }
+            if (i % 2 == 1) slice(s_cur, p_cur, grp);
+            if (i % 8 == 3) issue(dma_tile, (1 - PAR) * (LPT / 2) + i / 8);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        settle(s_cur, p_cur);
+    };
+    // tile (c + 1) / 2 must have landed before the scores of chunk c + 1 (c odd): at most the loads of the tile
+    // after it stay in flight; behind the barrier the stage of tile (c + 1) / 2 - 2 is free
+    auto tile_barrier = [&]() __attribute__((always_inline)) { asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(LPT) : "memory"); };
+
+    // tiles 0 and 1 and the K half of tile 2 (chunk 0 issues its V half); the V region that the second product
+    // of the first iteration reads (tile 3, with zero probabilities) must not hold NaN or infinity patterns
+    {
+        const half8_t z8 = {(half_t)0.f, (half_t)0.f, (half_t)0.f, (half_t)0.f, (half_t)0.f, (half_t)0.f, (half_t)0.f, (half_t)0.f};
+#pragma unroll
+        for (int i = 0; i < TILE / 8 / THREADS; ++i) store8(smem + VRING + 3 * TILE + (tid + THREADS * i) * 8, z8);
+    }
+#pragma unroll
+    for (int t = 0; t < LPT; ++t) issue(0, t);
+#pragma unroll
+    for (int t = 0; t < LPT; ++t) issue(clamp_tile(1), t);
+#pragma unroll
+    for (int t = 0; t < LPT / 2; ++t) issue(clamp_tile(2), t);
+    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(LPT + LPT / 2) : "memory");
+
+    // scores of chunk 0
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) {
+        const half8_t kf = load8(smem + klane[ks]);
+        if (ks == 0) asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(S[0]) : "v"(kf), "v"(qf[ks]));
+        else asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(S[0]) : "v"(kf), "v"(qf[ks]));
+    }
+    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+
+    // Two iterations per trip, so that the two score and probability sets keep their roles.  With an odd number
+    // of chunks the last iteration works on chunk nc, whose keys lie behind every query of the block: masked,
+    // its probabilities are zero, and the second product of the last real chunk rides on it.
+    int dma_tile = clamp_tile(2);
+    for (int c = 0; c < nc; c += 2) {
+        step(S[0], S[1], P[0], P[1], c, std::integral_constant<int, 0>{}, dma_tile);
+        tile_barrier();
+        dma_tile = clamp_tile(c / 2 + 3);
+        step(S[1], S[0], P[1], P[0], c + 1, std::integral_constant<int, 1>{}, dma_tile);
+    }
+    if (!(nc & 1)) { // second product of the last chunk
+        const int voff = (((nc - 1) >> 1) & 3) * TILE;
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                const half8_t vf = load8(smem + voff + vlane[1][u] + t * 2048);
+                asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(O[t]) : "v"(vf), "v"(pfrag(P[1], u)));
+            }
+    }
+    asm volatile("s_waitcnt vmcnt(0)\n\ts_nop 15\n\ts_nop 15" ::: "memory");
+
+    // O^T lane l: query q0w + l%32, dims 32 t + 8 (e/4) + 4 (l/32) + e%4
+    {
+        float lo, hi;
+        xhalf(l_run, lo, hi);
+        if (r < T) {
+            const float inv = 1.0f / (lo + hi);
+            half_t *orow = out + (size_t)r * ldo + (size_t)head * HD;
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+#pragma unroll
+                for (int e4 = 0; e4 < 4; ++e4) {
+                    half4_t v;
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) v[i] = (half_t)(O[t][4 * e4 + i] * inv);
+                    *reinterpret_cast<half4_t *>(orow + 32 * t + 8 * e4 + 4 * hb) = v;
+                }
+        }
+    }
+}
+
+static int launch_prefill_pipe(const half_t *q, int ldq, const half_t *kc, const half_t *vc, half_t *out, int ldo, int T,
+                               int pos0, int n_kv_heads, int max_pos, hipStream_t s) {
+    dim3 grid(n_kv_heads, (T + 63) / 64);
+    const size_t smem = 8 * 64 * 128 * sizeof(half_t); // four stages of a K and a V^T tile
+    auto kern = attn_prefill_pipe_kernel<4>;
+    static std::atomic<uint64_t> attr_done{0};
+    int rc = llm_ensure_max_smem((const void *)kern, smem, attr_done);
+    if (rc != LLM_OK) return rc;
+    kern<<<grid, dim3(512), smem, s>>>(q, ldq, kc, vc, out, ldo, T, pos0, max_pos);
+    LLM_LAUNCH_CHECK("attn_prefill_pipe_kernel");
+    return LLM_OK;
+}
+
 template <int HD, int G>
 static int launch_prefill(const half_t *q, int ldq, const half_t *kc, const half_t *vc, half_t *out, int ldo,
                           int T, int pos0, int n_kv_heads, int max_pos, hipStream_t s) {
@@ -369,6 +658,9 @@ extern "C" int llm_attn_prefill(const uint16_t *q, int ldq, const uint16_t *kc, 
     hipStream_t s = (hipStream_t)stream;
     const half_t *qp = (const half_t *)q, *kp = (const half_t *)kc, *vp = (const half_t *)vc;
     half_t *op = (half_t *)out;
+    // the pipelined kernel addresses one KV head's cache through a 32-bit buffer descriptor
+    if (head_dim == 128 && G == 4 && T >= AP_PIPE_MIN_ROWS && (size_t)max_pos * 128 * sizeof(half_t) < (1ull << 31))
+        return launch_prefill_pipe(qp, ldq, kp, vp, op, ldo, T, pos0, n_kv_heads, max_pos, s);
 #define AP_CASE(HD_, G_)                                                                        \
     if (head_dim == HD_ && G == G_)                                                             \
         return launch_prefill<HD_, G_>(qp, ldq, kp, vp, op, ldo, T, pos0, n_kv_heads, max_pos, s);

@@ -403,6 +403,39 @@ def test_attn_prefill(gpu, T, pos0, Hq, Hkv, hd):
     assert e <= TOL
 
 
+@pytest.mark.parametrize("T,pos0,shape", [(448, 0, "rising"), (448, 0, "falling"), (300, 37, "spikes"),
+                                          (448, 64, "flat")])
+def test_attn_prefill_score_ranges_that_move_the_softmax_reference(gpu, T, pos0, shape):
+    """The pipelined kernel (head size 128, group 4, 64 rows and more) keeps one softmax reference per query and
+    moves it only when a probability would overflow fp16.  Key magnitudes that rise along the sequence force that
+    move again and again; falling ones leave every later probability far below the reference; spikes put single
+    scores 2^30 above their neighbours; all-equal keys keep every probability at exactly 1."""
+    Hq, Hkv, hd = 32, 8, 128
+    P = pos0 + T
+    rng = np.random.default_rng(T + pos0)
+    q = rng.standard_normal((P, Hq * hd))
+    k = rng.standard_normal((P, Hkv * hd))
+    v = rng.standard_normal((P, Hkv * hd))
+    ramp = np.linspace(0.05, 6.0, P)[:, None]
+    if shape == "rising":
+        k *= ramp
+    elif shape == "falling":
+        k *= ramp[::-1]
+    elif shape == "spikes":
+        k[rng.integers(0, P, size=12)] *= 9.0
+    else:
+        k[:] = k[:1]
+    q, k, v = H.bits(q), H.bits(k), H.bits(v)
+    max_pos = (P + 63) // 64 * 64
+    kc, vc = gpu.ops.kv_layout(k, v, Hkv, hd, max_pos)
+    say("attn prefill", shape, T, pos0)
+    got = gpu.ops.attn_prefill(q[pos0:], kc, vc, pos0, Hq, Hkv, hd)
+    want = orc.attention(np.ascontiguousarray(q[pos0:]), k, v, pos0, Hq, Hkv, hd)
+    e = H.mixed_err(got, want)
+    say("  err", e, "max ulp", int(H.ulp_diff(got, want).max()))
+    assert e <= TOL
+
+
 def test_attn_prefill_8192_last_rows_and_uniform_key_property(gpu):
     T, Hq, Hkv, hd = 8192, 32, 8, 128
     q, k, v = _attn_inputs(11, T, Hq, Hkv, hd)
