@@ -744,6 +744,9 @@ __global__ __launch_bounds__(WGM * WGN * 64, OCC) void gemm_dma_kernel(const hal
 // activation and 8 weight fragments each, read during the sub-step before); the workgroup barrier sits between
 // the two: by then every wave has read the last fragments of the current stage and the next tile (issued
 // during the previous step's second sub-step, one load behind every fourth MFMA) must have landed.
+#ifndef DMA64_WIDE_EPILOGUE
+#define DMA64_WIDE_EPILOGUE 1 // 0: keep the 8-byte stores (for timing the two forms side by side)
+#endif
 template <int NB>
 __global__ __launch_bounds__(256, 1) void gemm_dma64_kernel(const half_t *__restrict__ x, int ldx, const half_t *__restrict__ w,
                                                            const half_t *__restrict__ w2, const half_t *res, int ldr,
@@ -878,6 +881,48 @@ __global__ __launch_bounds__(256, 1) void gemm_dma64_kernel(const half_t *__rest
 
     // lane l of a 16 x 16 block holds activation row l%16 and weight rows 4 (l/16) .. + 3: four output columns
     const int mrow = lane % 16, ncol0 = 4 * (lane / 16);
+    auto product = [&](int j, int i) { // the four fp16 results of weight block j, activation block i
+        half4_t h;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            if (NB == 2) h[e] = swiglu_to_half(acc[j][i][e], acc[4 + j][i][e]);
+            else h[e] = (half_t)acc[j][i][e];
+        }
+        return h;
+    };
+    // Wide form (every row of out and res 16-byte aligned): the lanes of rows 0/1 and 2/3 of the wave swap the
+    // results of two neighbouring weight blocks (v_permlane16_swap), after which a lane holds eight consecutive
+    // columns: 16-byte stores and residual loads that cover 64 contiguous bytes of a row per instruction instead
+    // of 8-byte ones that cover 32.  Same values, same roundings.
+    const bool wide = DMA64_WIDE_EPILOGUE && ((uintptr_t)out & 15u) == 0 && ldo % 8 == 0 && N % 8 == 0 &&
+                      (!(NB == 1 && res) || (((uintptr_t)res & 15u) == 0 && ldr % 8 == 0));
+    if (wide) {
+        const int g = lane / 16;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int m = m0 + wm * WTM + i * 16 + mrow;
+            const int mc = m < T ? m : T - 1;
+#pragma unroll
+            for (int jp = 0; jp < 4 / NB; ++jp) {
+                const uint2_t a = __builtin_bit_cast(uint2_t, product(2 * jp, i));
+                const uint2_t b = __builtin_bit_cast(uint2_t, product(2 * jp + 1, i));
+                // odd rows of the first operand <-> even rows of the second
+                const auto s0 = __builtin_amdgcn_permlane16_swap(a[0], b[0], false, false);
+                const auto s1 = __builtin_amdgcn_permlane16_swap(a[1], b[1], false, false);
+                const uint4_t packed = {s0[0], s1[0], s0[1], s1[1]};
+                half8_t h = __builtin_bit_cast(half8_t, packed);
+                const int n = n0 + (NB == 1 ? wn * 128 : wn * 64) + 16 * (2 * jp + (g & 1)) + 8 * (g >> 1);
+                if (NB == 1 && res) {
+                    const int nc = n < N ? n : N - 8;
+                    const half8_t rv = load8(res + (size_t)mc * ldr + nc);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) h[e] = (half_t)((float)h[e] + (float)rv[e]);
+                }
+                if (m < T && n < N) store8(out + (size_t)m * ldo + n, h);
+            }
+        }
+        return;
+    }
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
         const int m = m0 + wm * WTM + i * 16 + mrow;
@@ -885,18 +930,12 @@ __global__ __launch_bounds__(256, 1) void gemm_dma64_kernel(const half_t *__rest
 #pragma unroll
         for (int j = 0; j < 8 / NB; ++j) {
             const int n = n0 + (NB == 1 ? wn * 128 : wn * 64) + j * 16 + ncol0;
-            half4_t o;
+            half4_t o = product(j, i);
             if (NB == 1 && res) {
                 const int nc = n < N ? n : N - 4;
                 const half4_t rv = *reinterpret_cast<const half4_t *>(res + (size_t)mc * ldr + nc);
 #pragma unroll
-                for (int e = 0; e < 4; ++e) o[e] = (half_t)((float)(half_t)acc[j][i][e] + (float)rv[e]);
-            } else {
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    if (NB == 2) o[e] = swiglu_to_half(acc[j][i][e], acc[4 + j][i][e]);
-                    else o[e] = (half_t)acc[j][i][e];
-                }
+                for (int e = 0; e < 4; ++e) o[e] = (half_t)((float)o[e] + (float)rv[e]);
             }
             if (m < T && n < N) *reinterpret_cast<half4_t *>(out + (size_t)m * ldo + n) = o;
         }
