@@ -82,6 +82,9 @@ def main():
     ap.add_argument("--cpu-steps", type=int, default=8)
     ap.add_argument("--no-graph", action="store_true")
     ap.add_argument("--no-batch", action="store_true")
+    ap.add_argument("--no-api-loop", action="store_true",
+                    help="skip the three inference()-per-token legs (counter runs: thousands of launches less)")
+    ap.add_argument("--no-decode-8k", action="store_true", help="skip the 64 decode steps behind the 8192-token prompt")
     ap.add_argument("--ceiling", action="store_true",
                     help="instead of the benchmark: MFMA-only probe and the 8192-token pass with amd-smi power/clock samples")
     a = ap.parse_args()
@@ -134,11 +137,13 @@ def main():
         % (K, st.decode_ms, tok_s, 100 * frac, st.prefill_ms, wall))
 
     # ---- the reference's own loop: tokens_to_cuda once, then inference() per token (src/main.cu:109-123) ----
-    api = inference_api_loop(pkg, model, engine, cfg, prompt, 64)
-    api["sampling_candidates_on_device"] = inference_api_loop(pkg, model, engine, cfg, prompt, 64, "device")
-    api["sampling_on_host"] = inference_api_loop(pkg, model, engine, cfg, prompt, 64, "host")
-    log("inference() per token, as the reference's main loop drives it: %.1f tok/s (%.3f of llama3_generate)"
-        % (api["tok_per_s"], api["tok_per_s"] / tok_s))
+    api = None
+    if not a.no_api_loop:
+        api = inference_api_loop(pkg, model, engine, cfg, prompt, 64)
+        api["sampling_candidates_on_device"] = inference_api_loop(pkg, model, engine, cfg, prompt, 64, "device")
+        api["sampling_on_host"] = inference_api_loop(pkg, model, engine, cfg, prompt, 64, "host")
+        log("inference() per token, as the reference's main loop drives it: %.1f tok/s (%.3f of llama3_generate)"
+            % (api["tok_per_s"], api["tok_per_s"] / tok_s))
 
     # ---- dominant kernels against their rooflines (HIP events on their own stream) -------------
     roof = kernel_roofline(pkg, model, cfg)
@@ -165,13 +170,14 @@ def main():
         log("prefill 8192: %.1f ms -> %.0f tok/s (%.1f%% of fp16 MFMA peak)"
             % (ms8, T / sec, 100 * prefill["mfma_frac"]))
         # long-context decode (KV streaming next to weight streaming), 64 steps at ctx ~8.2K
-        engine.reset()
-        _, stl = engine.generate(p8k, 65)
-        ms_l = stl.decode_ms / stl.n_decode_steps
-        prefill["decode_at_8k"] = {"steps": stl.n_decode_steps, "ms_per_step": ms_l, "tok_per_s": 1e3 / ms_l,
-                                   "hbm_frac": decode_bytes(T + 33) * (1e3 / ms_l) / HBM_PEAK}
-        log("decode at ctx 8.2K: %.1f tok/s (%.1f%% of HBM roofline)"
-            % (1e3 / ms_l, 100 * prefill["decode_at_8k"]["hbm_frac"]))
+        if not a.no_decode_8k:
+            engine.reset()
+            _, stl = engine.generate(p8k, 65)
+            ms_l = stl.decode_ms / stl.n_decode_steps
+            prefill["decode_at_8k"] = {"steps": stl.n_decode_steps, "ms_per_step": ms_l, "tok_per_s": 1e3 / ms_l,
+                                       "hbm_frac": decode_bytes(T + 33) * (1e3 / ms_l) / HBM_PEAK}
+            log("decode at ctx 8.2K: %.1f tok/s (%.1f%% of HBM roofline)"
+                % (1e3 / ms_l, 100 * prefill["decode_at_8k"]["hbm_frac"]))
     engine.close()
 
     # ---- batched decode (beyond the reference, which serves one sequence): aggregate tokens/s --------
@@ -231,7 +237,7 @@ def main():
                                "decode steps, fp16 KV cache" % (a.prompt, K),
                    "prompt_tokens": a.prompt, "decode_steps": K, "graph": not a.no_graph},
         "decode_hbm_frac": frac, "decode_bytes_per_token": decode_bytes(ctx_avg),
-        "prompt_pass_ms": st.prefill_ms, "inference_api_tok_per_s": api["tok_per_s"], "inference_api": api,
+        "prompt_pass_ms": st.prefill_ms, "inference_api_tok_per_s": api["tok_per_s"] if api else None, "inference_api": api,
         "roofline": roof, "cpu_baseline": cpu, "prefill_8k": prefill, "batched_decode": batched,
         "first_tokens": [int(t) for t in toks[:8]],
     }
@@ -409,10 +415,10 @@ def prefill_kernel_roofline(pkg, model, cfg, T=8192):
     fl_a = 4.0 * hd * Hq * T * (T + 1) / 2
     for b in (x, hbuf, qkv, kc, vc, ao):
         b.free()
-    return {"kernel": "gemm_dma_kernel<2,2,2,4,true,1,4> = llm_linear_swiglu (gate/up + SiLU*mul, T=8192, N=2x14336, K=4096)",
+    return {"kernel": "gemm_dma64_kernel<2> = llm_linear_swiglu (gate/up + SiLU*mul, T=8192, N=2x14336, K=4096)",
             "bound": "mfma", "flops": fl_g, "avg_us": ms_g * 1e3, "achieved": fl_g / (ms_g * 1e-3) / 1e12,
             "peak": MFMA_F16_PEAK / 1e12, "unit": "TFLOP/s", "frac": fl_g / (ms_g * 1e-3) / MFMA_F16_PEAK,
-            "attention": {"kernel": "attn_prefill_kernel<128,4,2> = llm_attn_prefill (T=8192, 32/8 heads, causal)",
+            "attention": {"kernel": "attn_prefill_pipe_kernel<4> = llm_attn_prefill (T=8192, 32/8 heads, causal)",
                           "flops": fl_a, "avg_us": ms_a * 1e3, "achieved": fl_a / (ms_a * 1e-3) / 1e12,
                           "frac": fl_a / (ms_a * 1e-3) / MFMA_F16_PEAK}}
 

@@ -203,7 +203,10 @@ def test_linear_gemm_ragged_shapes(gpu, T, K, N):
     # 2..16 rows with K not a multiple of 1024: the skinny kernel that reads the weights through registers
     ("linear", 8, 768, 512, None), ("swiglu", 8, 768, 512, None),
     # gate/up with few output tiles and a long K at 64 and 128 rows: split k with the two-matrix reduction
-    ("swiglu", 64, 4096, 256, None), ("swiglu", 128, 4096, 256, None)])
+    ("swiglu", 64, 4096, 256, None), ("swiglu", 128, 4096, 256, None),
+    # the 256 x 256-tile kernel with output rows 8 but not 16 bytes apart: its 8-byte store epilogue (rows
+    # 16 bytes apart take 16-byte stores)
+    ("linear", 1100, 128, 10000, 10004), ("swiglu", 1030, 128, 5008, 5012)])
 def test_kernel_families_off_the_main_paths(gpu, what, T, K, N, ldo):
     """Shapes chosen so that every kernel family of the projections is launched by some test (the 8B shapes
     only reach the direct-to-LDS and skinny-DMA kernels)."""
@@ -386,6 +389,8 @@ def test_attn_decode_small_heads_and_gqa_map(gpu):
 
 @pytest.mark.parametrize("T,pos0,Hq,Hkv,hd", [(1, 0, 8, 2, 32), (16, 0, 8, 2, 32), (33, 7, 8, 2, 32),
                                               (64, 0, 32, 8, 128), (100, 60, 32, 8, 128), (512, 0, 32, 8, 128),
+                                              # fewer than 64 rows at the 8B head shape: the kernel of the short blocks
+                                              (40, 9, 32, 8, 128),
                                               # several pipelined tiles before the masked ones, rows not a multiple of the
                                               # block, prompt continued at an unaligned position; other group sizes and head dims
                                               (300, 37, 32, 8, 128), (257, 129, 8, 2, 64), (200, 300, 8, 1, 128),
