@@ -147,23 +147,45 @@ __device__ __forceinline__ void attn_decode_body(const AdArgs &a, float *sc, hal
     __syncthreads();
 
     // ---- 3. scores ---------------------------------------------------------------------
+    // On the matrix pipe: a block of 16 positions (NPB passes of this wavefront) against the G heads as columns
+    // 0..G-1 of a 16-column operand.  The K registers keep their row-contiguous load pattern (whole 256-byte rows
+    // per position); a wavefront turns a block into the MFMA's row operand through its own slice of LDS, with
+    // no workgroup barrier.  Lane (mg, mn) of the result holds rows 4 mg .. + 3 of the block for head mn.
     {
-        half8_t qreg[G];
+        constexpr int KS = HD / 32;   // k-steps of 32 dims
+        constexpr int NPB = 16 / PPW; // passes per block of 16 positions
+        constexpr int KLD = HD + 8;   // row stride of the staging slice (halves): fragment reads without bank conflicts
+        static_assert(KIT % NPB == 0 && G <= 16, "score blocks");
+        __shared__ __attribute__((aligned(16))) half_t kst_all[AD_WAVES * 16 * KLD];
+        half_t *kst = kst_all + wave * 16 * KLD;
+        const int mg = lane / 16, mn = lane % 16;
+        half8_t qreg[KS];
 #pragma unroll
-        for (int h = 0; h < G; ++h) qreg[h] = load8(qs + h * HD + sub * 8);
+        for (int ks = 0; ks < KS; ++ks)
+            qreg[ks] = mn < G ? load8(qs + mn * HD + 32 * ks + 8 * mg) : half8_t{0, 0, 0, 0, 0, 0, 0, 0};
         const float scale = 1.0f / sqrtf((float)HD);
 #pragma unroll
-        for (int it = 0; it < KIT; ++it) {
-            if (it * (AD_WAVES * PPW) + wave * PPW < len) { // wave-uniform: skip passes beyond the span
-                const int j = it * (AD_WAVES * PPW) + wave * PPW + lane / LPP;
-                half8_t kv = kreg[it];
-                if (FUSED && j == lpos) kv = load8(knew + sub * 8);
-                float part[G];
+        for (int b = 0; b < KIT / NPB; ++b) {
+            const int it0 = b * NPB;
+            if (it0 * (AD_WAVES * PPW) + wave * PPW < len) { // wave-uniform: skip blocks beyond the span
 #pragma unroll
-                for (int h = 0; h < G; ++h) part[h] = group_sum<LPP>(dot8(kv, qreg[h], 0.f));
-                if (sub == 0 && j < len) {
+                for (int q = 0; q < NPB; ++q) {
+                    const int j = (it0 + q) * (AD_WAVES * PPW) + wave * PPW + lane / LPP;
+                    half8_t kv = kreg[it0 + q];
+                    if (FUSED && j == lpos) kv = load8(knew + sub * 8);
+                    store8(kst + (q * PPW + lane / LPP) * KLD + sub * 8, kv);
+                }
+                float4_t acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                    for (int h = 0; h < G; ++h) sc[h * LS + j] = part[h] * scale;
+                for (int ks = 0; ks < KS; ++ks)
+                    acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(load8(kst + mn * KLD + 32 * ks + 8 * mg), qreg[ks], acc, 0, 0, 0);
+                if (mn < G) {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const int m = 4 * mg + i; // row of the block: pass m / PPW, position m % PPW of that pass
+                        const int j = (it0 + m / PPW) * (AD_WAVES * PPW) + wave * PPW + m % PPW;
+                        if (j < len) sc[mn * LS + j] = acc[i] * scale;
+                    }
                 }
             }
         }
