@@ -120,7 +120,10 @@ __global__ __launch_bounds__(AD_THREADS) void attn_oproj_kernel(const AdArgs a, 
     half8_t wreg[AO_ROWS][AO_KSTEPS];
     half_t resv[AO_ROWS];
     // a head start of about a microsecond for the attention's own loads (measured: 12.2 -> 11.4 us per launch)
-    for (int dl = 0; dl < 5; ++dl) __builtin_amdgcn_s_sleep(8);
+#ifndef AO_HEAD_START
+#define AO_HEAD_START 5
+#endif
+    for (int dl = 0; dl < AO_HEAD_START; ++dl) __builtin_amdgcn_s_sleep(8);
 #pragma unroll
     for (int r = 0; r < AO_ROWS; ++r) {
         int row = wslot + wtotal * r; // adjacent wavefronts read adjacent rows
@@ -164,18 +167,26 @@ __global__ __launch_bounds__(AD_THREADS) void attn_oproj_kernel(const AdArgs a, 
         }
     }
     __syncthreads();
+    // all rows of the wavefront against one read of the staged vector, then their reductions side by side
+    float acc[AO_ROWS];
+#pragma unroll
+    for (int r = 0; r < AO_ROWS; ++r) acc[r] = 0.f;
+#pragma unroll
+    for (int j = 0; j < AO_KSTEPS; ++j) {
+        const int k = lane * 8 + 512 * j;
+        if (k < K) {
+            const half8_t x = load8(xs + k);
+#pragma unroll
+            for (int r = 0; r < AO_ROWS; ++r) acc[r] = dot8(wreg[r][j], x, acc[r]);
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < AO_ROWS; ++r) acc[r] = wave_sum(acc[r]);
 #pragma unroll
     for (int r = 0; r < AO_ROWS; ++r) {
         const int row = wslot + wtotal * r;
-        float acc = 0.f;
-#pragma unroll
-        for (int j = 0; j < AO_KSTEPS; ++j) {
-            const int k = lane * 8 + 512 * j;
-            if (k < K) acc = dot8(wreg[r][j], load8(xs + k), acc);
-        }
-        acc = wave_sum(acc);
         if (lane == 0 && r < o.rows && row < N) {
-            half_t h = (half_t)acc;
+            half_t h = (half_t)acc[r];
             if (o.res) h = (half_t)((float)h + (float)resv[r]); // the reference's add_norm on the stored projection
             o.out[row] = h;
         }

@@ -39,52 +39,110 @@ struct AdArgs {
 #define AD_EMPTY16 0xFFFFu
 #define AD_POLL_LIMIT (1 << 18)
 
-template <int HD, int G, bool FUSED, int NDIM, int LS, bool TWOPASS = false, bool AGENT_OUT = false, bool POLL_IN = false>
-__device__ __forceinline__ void attn_decode_body(const AdArgs &a, float *sc, half_t *qs, half_t *knew, half_t *vnew,
-                                                 float *s_m, float *s_l, int *s_last, const int pos,
-                                                 const int n_active, const int split, const int d_begin,
-                                                 const bool appender, const int kvh_arg = -1, half_t *qkv_l = nullptr,
-                                                 int *timeouts = nullptr) {
-    constexpr int LPP = HD / 8;                    // lanes per position in the score pass
-    constexpr int PPW = 64 / LPP;                  // positions per wavefront pass
-    constexpr int KIT = LS / (AD_WAVES * PPW);  // K loads per thread
-    constexpr int DPW = NDIM / AD_WAVES;           // dims per wavefront in the P.V pass
-    static_assert(DPW >= 1, "too few dims for the workgroup");
-    constexpr int RR = DPW < 8 ? DPW : 8;          // dim rows per pass
-    constexpr int JL = 64 / RR;                    // lanes along positions (8, 16, 32 or 64)
-    constexpr int VP = DPW / RR;                   // passes over dims
-    constexpr int VIT = LS / (JL * 8);          // V loads per thread and pass
-    constexpr int HALF = HD / 2;
+// LDS of the attention.  The K staging buffer depends on the head size only: a kernel that instantiates the body
+// twice (for a quarter of the dims and for all of them) holds it once.
+template <int HD> __device__ __forceinline__ half_t *ad_lds_kst() {
+    __shared__ __attribute__((aligned(16))) half_t buf[AD_WAVES * 32 * (HD + 8)];
+    return buf;
+}
+template <int NDIM, int G> __device__ __forceinline__ float *ad_lds_ow() {
+    __shared__ __attribute__((aligned(16))) float buf[AD_WAVES * G * NDIM];
+    return buf;
+}
+template <int G> __device__ __forceinline__ float *ad_lds_ml() {
+    __shared__ float buf[AD_WAVES * G * 2];
+    return buf;
+}
 
-    const int kvh = kvh_arg >= 0 ? kvh_arg : (int)blockIdx.x, splits = a.splits;
+// One span of at most NB * 256 positions.  Wavefront w owns the 32-position blocks [256 c + 32 w, + 32), c < NB,
+// and runs the whole attention on them by itself, on the matrix pipe:
+//   scores   S[pos][head] = K_block . q^T    (v_mfma_f32_16x16x32_f16, K rows as the row operand, the group's
+//            queries as columns 0..G-1), with the K rows of the two 16-row halves interleaved so that a lane
+//            ends up with eight consecutive positions of one head: the layout of the next product's operand;
+//   softmax  relative to the wavefront's own maximum, in registers (reductions over four lanes);
+//   P.V      O[dim][head] += V_block^T . P   (the V cache is dim-major: a lane's operand is one 16-byte load).
+// What the wavefronts leave (maximum, sum, unnormalised O) is combined once through LDS.  Two workgroup barriers
+// in all, both on LDS contents only, so the cache-row loads stay in flight across the first.
+// Every cache-row load is issued unconditionally (positions beyond the span re-read its last row and are masked
+// afterwards): with a fixed number of loads in flight the waits can name the loads they need, and the rotation
+// of the new token, whose inputs are requested first, runs while the cache rows are still on their way.
+template <int HD, int G, bool FUSED, int NDIM, int LS, bool TWOPASS, bool AGENT_OUT, bool POLL_IN, int NB>
+__device__ __forceinline__ void attn_decode_span(const AdArgs &a, half_t *qs, half_t *knew, half_t *vnew,
+                                                 half_t *kst_all, float *ow_all, float *ml_all, const int pos,
+                                                 const int n_active, const int split, const int d_begin,
+                                                 const bool appender, const int kvh, half_t *qkv_l, int *timeouts) {
+    constexpr int LPP = HD / 8;   // lanes per K row
+    constexpr int PPW = 64 / LPP; // K rows per load instruction of a wavefront
+    constexpr int NPB = 32 / PPW; // load instructions per block
+    constexpr int KS = HD / 32;   // k-steps of the score product
+    constexpr int NT = NDIM / 16; // 16-dim tiles of the output
+    constexpr int KLD = HD + 8;   // row stride of the staging slice (halves): fragment reads without bank conflicts
+    constexpr int HALF = HD / 2;
+    static_assert(HD % 32 == 0 && NDIM % 16 == 0 && G <= 16 && NB * 256 <= LS, "attention tiling");
+    static_assert(G * HD <= AD_THREADS * 8 && G * NDIM / 4 <= AD_THREADS, "one staging / result item per thread");
+
+    const int splits = a.splits;
     const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
     const int max_pos = a.max_pos;
     const int ctx = pos + 1;
     const int s0 = split * LS;
     const int len = ctx - s0 < LS ? ctx - s0 : LS;
-    const int len_pad = (len + 63) / 64 * 64;
     half_t *kbase = a.kc + (size_t)kvh * max_pos * HD;
     half_t *vrow0 = a.vc + (size_t)kvh * HD * max_pos;
     const int lpos = pos - s0; // the new token inside this span (last span only)
+    const int mg = lane / 16, mn = lane % 16;
+    const int sub = lane % LPP, prow = lane / LPP;
+    const int blk0 = 32 * wave; // first position of this wavefront's block c is 256 c + blk0
 
-    // ---- 1. all K and V loads of the span ----------------------------------------
-    const int sub = lane % LPP;
-    half8_t kreg[KIT];
+    // ---- 0. the new token's inputs, requested before the cache rows -----------------------
+    constexpr int NRI = ((G + 1) * HALF + AD_THREADS - 1) / AD_THREADS; // rotation pairs per thread
+    constexpr int NVI = (HD + AD_THREADS - 1) / AD_THREADS;             // new-v elements per thread
+    constexpr bool EARLY = FUSED && !POLL_IN;
+    uint32_t pair_r[NRI];
+    float2_t cs_r[NRI];
+    half_t vnew_r[NVI];
+    half8_t q_r = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+    if (EARLY) {
+        const int Hq = a.n_kv_heads * G;
+        const float *cs = a.table + (size_t)pos * HALF * 2;
 #pragma unroll
-    for (int it = 0; it < KIT; ++it) {
-        const int j = it * (AD_WAVES * PPW) + wave * PPW + lane / LPP;
-        kreg[it] = j < len ? load8(kbase + (size_t)(s0 + j) * HD + sub * 8) : half8_t{0, 0, 0, 0, 0, 0, 0, 0};
-    }
-    const int rr = lane / JL, jc = lane % JL;
-    half8_t vreg[VP][VIT];
-#pragma unroll
-    for (int p = 0; p < VP; ++p) {
-        const int d = d_begin + wave * DPW + p * RR + rr;
-#pragma unroll
-        for (int it = 0; it < VIT; ++it) {
-            const int j = (jc + JL * it) * 8;
-            vreg[p][it] = j < len ? load8(vrow0 + (size_t)d * max_pos + s0 + j) : half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+        for (int r = 0; r < NRI; ++r) {
+            const int p = tid + r * AD_THREADS;
+            if (p < (G + 1) * HALF) {
+                const int h = p / HALF, i = p % HALF; // h == G: the new key
+                const half_t *src = h < G ? a.q + (size_t)(kvh * G + h) * HD + 2 * i
+                                          : a.q + (size_t)Hq * HD + (size_t)kvh * HD + 2 * i;
+                pair_r[r] = *reinterpret_cast<const uint32_t *>(src);
+                cs_r[r] = *reinterpret_cast<const float2_t *>(cs + 2 * i);
+            }
         }
+#pragma unroll
+        for (int r = 0; r < NVI; ++r) {
+            const int d = tid + r * AD_THREADS;
+            if (d < HD) vnew_r[r] = a.q[(size_t)(Hq + a.n_kv_heads) * HD + (size_t)kvh * HD + d];
+        }
+    }
+    if (!FUSED && tid * 8 < G * HD) q_r = load8(a.q + (size_t)kvh * G * HD + tid * 8);
+
+    // ---- 1. every K and V load of the wavefront's blocks -----------------------------------
+    half8_t kreg[NB][NPB];
+#pragma unroll
+    for (int c = 0; c < NB; ++c) {
+#pragma unroll
+        for (int q = 0; q < NPB; ++q) {
+            const int j = 256 * c + blk0 + q * PPW + prow;
+            const int jc = j < len ? j : len - 1;
+            kreg[c][q] = load8(kbase + (size_t)(s0 + jc) * HD + sub * 8);
+        }
+    }
+    half8_t vreg[NB][NT]; // lane (mg, mn): dim 16 t + mn, positions 8 mg .. + 7 of the block
+#pragma unroll
+    for (int c = 0; c < NB; ++c) {
+        const int j = 256 * c + blk0 + 8 * mg;
+        const int jc = j < len ? j : ((len - 1) & ~7);
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+            vreg[c][t] = load8(vrow0 + (size_t)(d_begin + 16 * t + mn) * max_pos + s0 + jc);
     }
 
     // ---- 2. queries into LDS; fused: rotate them and the new K, append K/V ---------
@@ -114,182 +172,203 @@ __device__ __forceinline__ void attn_decode_body(const AdArgs &a, float *sc, hal
             }
             __syncthreads();
         }
-        for (int p = tid; p < (G + 1) * HALF; p += AD_THREADS) {
-            const int h = p / HALF, i = p % HALF; // h == G: the new key
-            const half_t *src = POLL_IN ? qkv_l + (size_t)h * HD + 2 * i
-                                : h < G ? qkv + (size_t)(kvh * G + h) * HD + 2 * i
-                                        : qkv + (size_t)Hq * HD + (size_t)kvh * HD + 2 * i;
-            const float c = cs[2 * i], sn = cs[2 * i + 1];
-            const float e = (float)src[0], o = (float)src[1];
-            const float ce = c * e, so = sn * o, se = sn * e, co = c * o;
-            const half_t re = (half_t)(ce - so), ro = (half_t)(se + co);
-            if (h < G) {
-                qs[h * HD + 2 * i] = re;
-                qs[h * HD + 2 * i + 1] = ro;
-            } else {
-                knew[2 * i] = re;
-                knew[2 * i + 1] = ro;
-                if (appender) {
-                    kbase[(size_t)pos * HD + 2 * i] = re;
-                    kbase[(size_t)pos * HD + 2 * i + 1] = ro;
+#pragma unroll
+        for (int r = 0; r < NRI; ++r) {
+            const int p = tid + r * AD_THREADS;
+            if (p < (G + 1) * HALF) {
+                const int h = p / HALF, i = p % HALF; // h == G: the new key
+                float c, sn, e, o;
+                if (EARLY) {
+                    const half2_t pr = __builtin_bit_cast(half2_t, pair_r[r]);
+                    c = cs_r[r][0], sn = cs_r[r][1], e = (float)pr[0], o = (float)pr[1];
+                } else {
+                    const half_t *src = qkv_l + (size_t)h * HD + 2 * i;
+                    c = cs[2 * i], sn = cs[2 * i + 1], e = (float)src[0], o = (float)src[1];
+                }
+                const float ce = c * e, so = sn * o, se = sn * e, co = c * o;
+                const half_t re = (half_t)(ce - so), ro = (half_t)(se + co);
+                if (h < G) {
+                    qs[h * HD + 2 * i] = re;
+                    qs[h * HD + 2 * i + 1] = ro;
+                } else {
+                    knew[2 * i] = re;
+                    knew[2 * i + 1] = ro;
+                    if (appender) {
+                        kbase[(size_t)pos * HD + 2 * i] = re;
+                        kbase[(size_t)pos * HD + 2 * i + 1] = ro;
+                    }
                 }
             }
         }
-        const half_t *vsrc = POLL_IN ? qkv_l + (size_t)(G + 1) * HD : qkv + (size_t)(Hq + a.n_kv_heads) * HD + (size_t)kvh * HD;
-        for (int d = tid; d < HD; d += AD_THREADS) {
-            const half_t v = vsrc[d];
-            vnew[d] = v;
-            if (appender) vrow0[(size_t)d * max_pos + pos] = v;
+#pragma unroll
+        for (int r = 0; r < NVI; ++r) {
+            const int d = tid + r * AD_THREADS;
+            if (d < HD) {
+                const half_t v = EARLY ? vnew_r[r] : qkv_l[(size_t)(G + 1) * HD + d];
+                vnew[d] = v;
+                if (appender) vrow0[(size_t)d * max_pos + pos] = v;
+            }
         }
     } else {
-        for (int c = tid * 8; c < G * HD; c += AD_THREADS * 8) store8(qs + c, load8(a.q + (size_t)kvh * G * HD + c));
+        if (tid * 8 < G * HD) store8(qs + tid * 8, q_r);
     }
-    __syncthreads();
+    // This barrier guards LDS contents only (queries, new key and value): it waits for the LDS writes and leaves
+    // the cache-row loads in flight, which __syncthreads() would drain first.
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 
-    // ---- 3. scores ---------------------------------------------------------------------
-    // On the matrix pipe: a block of 16 positions (NPB passes of this wavefront) against the G heads as columns
-    // 0..G-1 of a 16-column operand.  The K registers keep their row-contiguous load pattern (whole 256-byte rows
-    // per position); a wavefront turns a block into the MFMA's row operand through its own slice of LDS, with
-    // no workgroup barrier.  Lane (mg, mn) of the result holds rows 4 mg .. + 3 of the block for head mn.
-    {
-        constexpr int KS = HD / 32;   // k-steps of 32 dims
-        constexpr int NPB = 16 / PPW; // passes per block of 16 positions
-        constexpr int KLD = HD + 8;   // row stride of the staging slice (halves): fragment reads without bank conflicts
-        static_assert(KIT % NPB == 0 && G <= 16, "score blocks");
-        __shared__ __attribute__((aligned(16))) half_t kst_all[AD_WAVES * 16 * KLD];
-        half_t *kst = kst_all + wave * 16 * KLD;
-        const int mg = lane / 16, mn = lane % 16;
-        half8_t qreg[KS];
+    // ---- 3. scores of this wavefront's blocks -------------------------------------------
+    // The K registers keep the row-contiguous load pattern (whole rows per position); the wavefront turns a block
+    // into the MFMA's row operand through its own slice of LDS.  Row m of half u of the product is block row
+    // 8 (m / 4) + 4 u + m % 4, so that lane (mg, mn) ends up with positions 8 mg .. + 7 of the block for head mn.
+    half_t *kst = kst_all + wave * 32 * KLD;
+    half8_t qreg[KS];
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks)
-            qreg[ks] = mn < G ? load8(qs + mn * HD + 32 * ks + 8 * mg) : half8_t{0, 0, 0, 0, 0, 0, 0, 0};
-        const float scale = 1.0f / sqrtf((float)HD);
+    for (int ks = 0; ks < KS; ++ks)
+        qreg[ks] = mn < G ? load8(qs + mn * HD + 32 * ks + 8 * mg) : half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+    const float scale = 1.0f / sqrtf((float)HD);
+    float sv[NB][8];
 #pragma unroll
-        for (int b = 0; b < KIT / NPB; ++b) {
-            const int it0 = b * NPB;
-            if (it0 * (AD_WAVES * PPW) + wave * PPW < len) { // wave-uniform: skip blocks beyond the span
+    for (int c = 0; c < NB; ++c) {
 #pragma unroll
-                for (int q = 0; q < NPB; ++q) {
-                    const int j = (it0 + q) * (AD_WAVES * PPW) + wave * PPW + lane / LPP;
-                    half8_t kv = kreg[it0 + q];
-                    if (FUSED && j == lpos) kv = load8(knew + sub * 8);
-                    store8(kst + (q * PPW + lane / LPP) * KLD + sub * 8, kv);
-                }
-                float4_t acc = {0.f, 0.f, 0.f, 0.f};
+        for (int q = 0; q < NPB; ++q) {
+            const int r = q * PPW + prow;
+            half8_t kv = kreg[c][q];
+            if (FUSED && 256 * c + blk0 + r == lpos) kv = load8(knew + sub * 8);
+            store8(kst + r * KLD + sub * 8, kv);
+        }
 #pragma unroll
-                for (int ks = 0; ks < KS; ++ks)
-                    acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(load8(kst + mn * KLD + 32 * ks + 8 * mg), qreg[ks], acc, 0, 0, 0);
-                if (mn < G) {
+        for (int u = 0; u < 2; ++u) {
+            const int row = 8 * (mn / 4) + 4 * u + mn % 4;
+            float4_t acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        const int m = 4 * mg + i; // row of the block: pass m / PPW, position m % PPW of that pass
-                        const int j = (it0 + m / PPW) * (AD_WAVES * PPW) + wave * PPW + m % PPW;
-                        if (j < len) sc[mn * LS + j] = acc[i] * scale;
-                    }
-                }
+            for (int ks = 0; ks < KS; ++ks)
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(load8(kst + row * KLD + 32 * ks + 8 * mg), qreg[ks], acc, 0, 0, 0);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int j = 256 * c + blk0 + 8 * mg + 4 * u + i;
+                sv[c][4 * u + i] = j < len ? acc[i] * scale : -FLT_MAX;
             }
         }
     }
-    __syncthreads();
 
-    // ---- 4. local softmax statistics: wavefront w takes heads w, w+8, ... ------------------
-    for (int h = wave; h < G; h += AD_WAVES) {
-        float *row = sc + h * LS;
-        float mx = -FLT_MAX;
-        for (int j = lane; j < len; j += 64) mx = fmaxf(mx, row[j]);
-        mx = wave_max(mx);
-        float sum = 0.f;
-        for (int j = lane; j < len_pad; j += 64) {
-            float e = j < len ? expf(row[j] - mx) : 0.f;
-            row[j] = e;
-            sum += e;
-        }
-        sum = wave_sum(sum);
-        if (lane == 0) {
-            s_m[h] = mx;
-            s_l[h] = sum;
+    // ---- 4. softmax relative to the wavefront's own maximum ------------------------------
+    float m_w = -FLT_MAX;
+#pragma unroll
+    for (int c = 0; c < NB; ++c)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) m_w = fmaxf(m_w, sv[c][e]);
+    m_w = rows_max(m_w);
+    float l_w = 0.f;
+    half8_t pf[NB];
+#pragma unroll
+    for (int c = 0; c < NB; ++c) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const int j = 256 * c + blk0 + 8 * mg + e;
+            const float p = j < len ? __expf(sv[c][e] - m_w) : 0.f;
+            l_w += p;
+            pf[c][e] = (half_t)p;
         }
     }
-    __syncthreads();
+    l_w = rows_sum(l_w);
 
-    // ---- 5. unnormalised P.V from the registers ----------------------------------------------
+    // ---- 5. unnormalised P.V of the blocks -------------------------------------------------
+    float *ow = ow_all + wave * G * NDIM;
 #pragma unroll
-    for (int p = 0; p < VP; ++p) {
-        const int d = d_begin + wave * DPW + p * RR + rr;
-        float acc[G];
+    for (int t = 0; t < NT; ++t) {
+        float4_t o = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int h = 0; h < G; ++h) acc[h] = 0.f;
+        for (int c = 0; c < NB; ++c) {
+            const int j = 256 * c + blk0 + 8 * mg;
+            half8_t vf = vreg[c][t];
+            if (FUSED && lpos >= j && lpos < j + 8) { // the chunk that holds the new token
+                const half_t vn = vnew[d_begin + 16 * t + mn];
 #pragma unroll
-        for (int it = 0; it < VIT; ++it) {
-            const int j = (jc + JL * it) * 8;
-            if (j < len) {
-                float vf[8];
-#pragma unroll
-                for (int i = 0; i < 8; ++i) vf[i] = (float)vreg[p][it][i];
-                if (FUSED && lpos >= j && lpos < j + 8) { // the chunk that holds the new token (rare)
-                    const float vn = (float)vnew[d];
-#pragma unroll
-                    for (int i = 0; i < 8; ++i) vf[i] = (j + i == lpos) ? vn : vf[i];
-                }
-                if (j + 8 > len) { // the chunk that straddles the end of the span (rare)
-#pragma unroll
-                    for (int i = 0; i < 8; ++i) vf[i] = (j + i < len) ? vf[i] : 0.f;
-                }
-#pragma unroll
-                for (int h = 0; h < G; ++h) {
-                    const float *e = sc + h * LS + j;
-#pragma unroll
-                    for (int i = 0; i < 8; ++i) acc[h] = fmaf(e[i], vf[i], acc[h]);
-                }
+                for (int e = 0; e < 8; ++e) vf[e] = (j + e == lpos) ? vn : vf[e];
             }
-        }
+            if (j + 8 > len) { // beyond or across the end of the span
 #pragma unroll
-        for (int h = 0; h < G; ++h) {
-            if (JL <= 16) {
-                acc[h] = group_sum<(JL <= 16 ? JL : 16)>(acc[h]);
+                for (int e = 0; e < 8; ++e) vf[e] = (j + e < len) ? vf[e] : (half_t)0.f;
+            }
+            o = __builtin_amdgcn_mfma_f32_16x16x32_f16(vf, pf[c], o, 0, 0, 0);
+        }
+        if (mn < G) *reinterpret_cast<float4_t *>(ow + mn * NDIM + 16 * t + 4 * mg) = o; // dims 16 t + 4 mg .. + 3
+    }
+    if (mn < G && mg == 0) {
+        ml_all[(wave * G + mn) * 2] = m_w;
+        ml_all[(wave * G + mn) * 2 + 1] = l_w;
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+
+    // ---- 6. the wavefronts' parts into one: four dims of one head per thread ---------------------
+    if (tid < G * NDIM / 4) {
+        const int h = tid / (NDIM / 4), d4 = tid % (NDIM / 4);
+        float mw[AD_WAVES];
+        float M = -FLT_MAX;
+#pragma unroll
+        for (int w = 0; w < AD_WAVES; ++w) {
+            mw[w] = ml_all[(w * G + h) * 2];
+            M = fmaxf(M, mw[w]);
+        }
+        float L = 0.f;
+        float4_t O = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int w = 0; w < AD_WAVES; ++w) {
+            const float f = __expf(mw[w] - M); // 0 for a wavefront without a position of the span
+            L += f * ml_all[(w * G + h) * 2 + 1];
+            const float4_t part = *reinterpret_cast<const float4_t *>(ow_all + (w * G + h) * NDIM + 4 * d4);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) O[i] += f * part[i];
+        }
+        if (n_active == 1 && !TWOPASS) {
+            half_t *dst = a.out + (size_t)(kvh * G + h) * HD + d_begin + 4 * d4;
+            if (AGENT_OUT) {
+                // 8-byte device-scope stores (written through to the point where every XCD reads them): 2-byte
+                // write-through stores cost a read-modify-write each
+                unsigned long long v = 0ull;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    uint16_t bits = __builtin_bit_cast(uint16_t, (half_t)(O[i] / L));
+                    if (bits == 0xFFFFu) bits = 0xFFFEu; // 0xFFFF marks "not written yet" for the reader
+                    v |= (unsigned long long)bits << (16 * i);
+                }
+                __hip_atomic_store(reinterpret_cast<unsigned long long *>(dst), v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             } else {
-                acc[h] = group_sum<16>(acc[h]);
-                acc[h] += __shfl_xor(acc[h], 16);
-                if (JL == 64) acc[h] += __shfl_xor(acc[h], 32);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) dst[i] = (half_t)(O[i] / L);
             }
-        }
-        if (jc == 0) {
-            if (n_active == 1 && !TWOPASS) {
+        } else {
+            float *dst = a.ws_acc + (((size_t)kvh * splits + split) * G + h) * HD + d_begin + 4 * d4;
 #pragma unroll
-                for (int h = 0; h < G; ++h) {
-                    const half_t r = (half_t)(acc[h] / s_l[h]);
-                    if (AGENT_OUT) { // collected in LDS (the queries are no longer needed), stored wide below
-                        uint16_t bits = __builtin_bit_cast(uint16_t, r);
-                        if (bits == 0xFFFFu) bits = 0xFFFEu; // 0xFFFF marks "not written yet" for the reader
-                        reinterpret_cast<uint16_t *>(qs)[h * NDIM + (d - d_begin)] = bits;
-                    }
-                    else
-                        a.out[(size_t)(kvh * G + h) * HD + d] = r;
-                }
-            } else {
-#pragma unroll
-                for (int h = 0; h < G; ++h) a.ws_acc[(((size_t)kvh * splits + split) * G + h) * HD + d] = acc[h];
+            for (int i = 0; i < 4; ++i) dst[i] = O[i];
+            if (d4 == 0) {
+                a.ws_ml[(((size_t)kvh * splits + split) * G + h) * 2 + 0] = M;
+                a.ws_ml[(((size_t)kvh * splits + split) * G + h) * 2 + 1] = L;
             }
         }
     }
-    if (AGENT_OUT) {
-        // This workgroup's G x NDIM results go out as 8-byte device-scope stores (written through to the
-        // point where every XCD reads them): 2-byte write-through stores cost a read-modify-write each.
-        static_assert(!AGENT_OUT || NDIM % 4 == 0, "results are stored four at a time");
-        __syncthreads();
-        if (tid < G * NDIM / 4) {
-            const int h = tid / (NDIM / 4), q = tid % (NDIM / 4);
-            const unsigned long long v = reinterpret_cast<const unsigned long long *>(qs)[tid];
-            __hip_atomic_store(reinterpret_cast<unsigned long long *>(a.out + (size_t)(kvh * G + h) * HD + d_begin) + q, v,
-                               __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
-    }
+}
+
+template <int HD, int G, bool FUSED, int NDIM, int LS, bool TWOPASS = false, bool AGENT_OUT = false, bool POLL_IN = false>
+__device__ __forceinline__ void attn_decode_body(const AdArgs &a, float *sc, half_t *qs, half_t *knew, half_t *vnew,
+                                                 float *s_m, float *s_l, int *s_last, const int pos,
+                                                 const int n_active, const int split, const int d_begin,
+                                                 const bool appender, const int kvh_arg = -1, half_t *qkv_l = nullptr,
+                                                 int *timeouts = nullptr) {
+    static_assert(LS == 256 || LS == 512, "span length");
+    half_t *kst_all = ad_lds_kst<HD>();  // K blocks, one slice per wavefront
+    float *ow_all = ad_lds_ow<NDIM, G>();  // unnormalised P.V per wavefront
+    float *ml_all = ad_lds_ml<G>();      // (max, sum) per wavefront and head
+    const int kvh = kvh_arg >= 0 ? kvh_arg : (int)blockIdx.x, splits = a.splits;
+    const int tid = threadIdx.x;
+    // one or two blocks per wavefront, each form with its own fixed number of loads in flight
+    if (LS == 512 && pos + 1 - split * LS > 256)
+        attn_decode_span<HD, G, FUSED, NDIM, LS, TWOPASS, AGENT_OUT, POLL_IN, LS / 256>(
+            a, qs, knew, vnew, kst_all, ow_all, ml_all, pos, n_active, split, d_begin, appender, kvh, qkv_l, timeouts);
+    else
+        attn_decode_span<HD, G, FUSED, NDIM, LS, TWOPASS, AGENT_OUT, POLL_IN, 1>(
+            a, qs, knew, vnew, kst_all, ow_all, ml_all, pos, n_active, split, d_begin, appender, kvh, qkv_l, timeouts);
     if (n_active == 1 && !TWOPASS) return;
-    if (tid < G) {
-        a.ws_ml[(((size_t)kvh * splits + split) * G + tid) * 2 + 0] = s_m[tid];
-        a.ws_ml[(((size_t)kvh * splits + split) * G + tid) * 2 + 1] = s_l[tid];
-    }
-
     if (TWOPASS) return; // attn_merge_kernel combines the spans
 
     // ---- 6. the last workgroup of this head merges the spans ------------------------------------

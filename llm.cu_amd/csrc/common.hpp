@@ -11,6 +11,7 @@ typedef _Float16 half_t;
 typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
 typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef float float2_t __attribute__((ext_vector_type(2)));
 typedef float float4_t __attribute__((ext_vector_type(4)));
 typedef float float16_t __attribute__((ext_vector_type(16)));
 typedef uint32_t uint4_t __attribute__((ext_vector_type(4)));
@@ -103,19 +104,29 @@ template <int N> __device__ __forceinline__ float group_max(float v) {
     return v;
 }
 
-__device__ __forceinline__ float wave_sum(float v) {
-    v = group_sum<16>(v);
-    v += __shfl_xor(v, 16);
-    v += __shfl_xor(v, 32);
-    return v;
+// max / sum over the lanes l, l ^ 16, l ^ 32, l ^ 48 (one lane of each 16-lane row); every lane gets the result.
+// Two swaps between rows (v_permlane16_swap, v_permlane32_swap) instead of two trips through the LDS crossbar
+// (ds_bpermute); the operands meet in the same order as with __shfl_xor(v, 16) followed by __shfl_xor(v, 32).
+__device__ __forceinline__ float rows_max(float v) {
+    uint32_t x = __builtin_bit_cast(uint32_t, v);
+    const auto a = __builtin_amdgcn_permlane16_swap(x, x, false, false); // rows (0,0,2,2) and (1,1,3,3)
+    v = fmaxf(__builtin_bit_cast(float, (uint32_t)a[0]), __builtin_bit_cast(float, (uint32_t)a[1]));
+    x = __builtin_bit_cast(uint32_t, v);
+    const auto b = __builtin_amdgcn_permlane32_swap(x, x, false, false); // halves (lo,lo) and (hi,hi)
+    return fmaxf(__builtin_bit_cast(float, (uint32_t)b[0]), __builtin_bit_cast(float, (uint32_t)b[1]));
+}
+__device__ __forceinline__ float rows_sum(float v) {
+    uint32_t x = __builtin_bit_cast(uint32_t, v);
+    const auto a = __builtin_amdgcn_permlane16_swap(x, x, false, false);
+    v = __builtin_bit_cast(float, (uint32_t)a[0]) + __builtin_bit_cast(float, (uint32_t)a[1]);
+    x = __builtin_bit_cast(uint32_t, v);
+    const auto b = __builtin_amdgcn_permlane32_swap(x, x, false, false);
+    return __builtin_bit_cast(float, (uint32_t)b[0]) + __builtin_bit_cast(float, (uint32_t)b[1]);
 }
 
-__device__ __forceinline__ float wave_max(float v) {
-    v = group_max<16>(v);
-    v = fmaxf(v, __shfl_xor(v, 16));
-    v = fmaxf(v, __shfl_xor(v, 32));
-    return v;
-}
+__device__ __forceinline__ float wave_sum(float v) { return rows_sum(group_sum<16>(v)); }
+
+__device__ __forceinline__ float wave_max(float v) { return rows_max(group_max<16>(v)); }
 
 // 8 fp16 x 8 fp16 -> fp32, accumulated with v_dot2_f32_f16.
 __device__ __forceinline__ float dot8(half8_t a, half8_t b, float acc) {
