@@ -6,8 +6,9 @@
 // over elements 4i..4i+3, then s[i] += s[i + off] for off = n/2, n/4, ..., 1
 // over the n = d/4 partials.  That tree reduces the index bits from the top
 // down, so a workgroup of THREADS threads holds slots i = t + THREADS*j in
-// thread t, folds j in registers first (the top bits), then folds the thread
-// index through LDS down to one wavefront and finishes with lane shuffles.
+// thread t, folds j in registers first (the top bits), then the wavefront index
+// (every wavefront for itself, from one exchange through LDS) and finishes with
+// swaps and shifts between lanes.
 // fp32 addition is commutative, so which side of a pair a value sits on does
 // not matter; the association is the reference's, hence so are the bits.
 #pragma once
@@ -49,6 +50,24 @@ __device__ __forceinline__ void rms_load(const half_t *__restrict__ xrow, const 
     }
 }
 
+// Lane bits 5..0 of the tree, in that order: lane l takes the value of lane l + off for off = 32, 16, 8, 4, 2, 1, so
+// lane 0 ends with the reference's association; every lane of the wavefront gets that value.  The two steps
+// across 16-lane rows are register swaps (v_permlane32_swap, v_permlane16_swap: both halves of a pair compute
+// the same sum, addition being commutative), the four inside a row are DPP row shifts: no trip through LDS.
+__device__ __forceinline__ float rms_fold_lanes(float v) {
+    uint32_t x = __builtin_bit_cast(uint32_t, v);
+    const auto a = __builtin_amdgcn_permlane32_swap(x, x, false, false); // (lo, lo) and (hi, hi)
+    v = __builtin_bit_cast(float, (uint32_t)a[0]) + __builtin_bit_cast(float, (uint32_t)a[1]);
+    x = __builtin_bit_cast(uint32_t, v);
+    const auto b = __builtin_amdgcn_permlane16_swap(x, x, false, false); // rows (0,0,2,2) and (1,1,3,3)
+    v = __builtin_bit_cast(float, (uint32_t)b[0]) + __builtin_bit_cast(float, (uint32_t)b[1]);
+    v += dpp_move<0x108>(v); // row_shl:8 (lanes shifted in from beyond the row read as 0)
+    v += dpp_move<0x104>(v); // row_shl:4
+    v += dpp_move<0x102>(v); // row_shl:2
+    v += dpp_move<0x101>(v); // row_shl:1
+    return __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, v)));
+}
+
 // Sum of squares of the loaded row in the reference's order; every thread gets it.
 template <int THREADS, int MAXR>
 __device__ __forceinline__ float rms_sum_squares(const RmsRow<MAXR> &r, int d, float *red, const int t = threadIdx.x) {
@@ -76,26 +95,23 @@ __device__ __forceinline__ float rms_sum_squares(const RmsRow<MAXR> &r, int d, f
     }
     float v = p[0];
     if (THREADS > 64) {
+        // thread-index bits above the lane: every wavefront reads the partial of its lane position in each
+        // wavefront and folds them top-down itself (one barrier; no wavefront waits for another's fold)
+        constexpr int W = THREADS / 64;
         red[t] = v;
         __syncthreads();
-        for (int off = THREADS / 2; off >= 64; off >>= 1) {
-            if (t < off) red[t] += red[t + off];
-            __syncthreads();
-        }
-        v = red[t & 63]; // wave 0 holds the live values; other waves read them too (unused)
-    }
-    // lane bits 5..0, in that order; lane 0 of wave 0 ends with the reference's sum
+        float w[W];
 #pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) v += __shfl_down(v, off);
-    if (THREADS > 64) {
-        __syncthreads();
-        if (t == 0) red[THREADS] = v;
-        __syncthreads();
-        v = red[THREADS];
-    } else {
-        v = __shfl(v, 0);
+        for (int k = 0; k < W; ++k) w[k] = red[(t & 63) + 64 * k];
+#pragma unroll
+        for (int off = W / 2; off >= 1; off >>= 1) {
+#pragma unroll
+            for (int k = 0; k < (W > 1 ? W / 2 : 1); ++k)
+                if (k < off) w[k] += w[k + off];
+        }
+        v = w[0];
     }
-    return v;
+    return rms_fold_lanes(v);
 }
 
 // rms = sqrtf((float)(eps + (double)(ss / d))), the double add as in the
