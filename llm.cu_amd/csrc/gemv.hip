@@ -39,6 +39,10 @@ struct GemvArgs {
 template <int MODE>
 __global__ __launch_bounds__(GEMV_THREADS) void gemv_kernel(const GemvArgs a) {
     constexpr int NW = MODE == GV_SWIGLU ? 2 : 1; // weight streams per row
+#ifndef GEMV_NBUF1
+#define GEMV_NBUF1 2
+#endif
+    constexpr int NBUF = NW == 2 ? 2 : GEMV_NBUF1; // steps in flight per wavefront (2 KB per stream and step)
     extern __shared__ __attribute__((aligned(16))) half_t xs[];
     __shared__ float red[GEMV_THREADS + 1];
     __shared__ unsigned long long best[GEMV_WAVES];
@@ -52,7 +56,7 @@ __global__ __launch_bounds__(GEMV_THREADS) void gemv_kernel(const GemvArgs a) {
     const int spr = (K + GEMV_SPAN - 1) / GEMV_SPAN; // spans per row
     const int steps = a.rpw * spr;
 
-    half8_t buf[2][NW][GEMV_U];
+    half8_t buf[NBUF][NW][GEMV_U];
     // loads of step s (row i = s / spr, span s % spr) into buf[which]
     auto issue = [&](int which, int i, int sp) {
         int row = row_base + row_step * i;
@@ -76,21 +80,24 @@ __global__ __launch_bounds__(GEMV_THREADS) void gemv_kernel(const GemvArgs a) {
         }
     };
 
-    // the activation loads go out first, then two steps of weights; only then
+    // the activation loads go out first, then NBUF steps of weights; only then
     // does anything wait (the norm's reduction), so HBM is busy throughout
     RmsRow<GEMV_NORM_R> xr;
-    half8_t xraw[4];
+#ifndef GEMV_XRAW
+#define GEMV_XRAW 8
+#endif
+    half8_t xraw[GEMV_XRAW]; // the first GEMV_XRAW * 2048 elements of a plain input vector, asked for before the weights
     if (a.gain) {
         rms_load<GEMV_THREADS, GEMV_NORM_R>(a.x, a.gain, K, xr);
     } else {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
+        for (int j = 0; j < GEMV_XRAW; ++j) {
             const int c = (threadIdx.x + GEMV_THREADS * j) * 8;
             if (c < K) xraw[j] = load8(a.x + c);
         }
     }
-    issue_next(0);
-    issue_next(1);
+#pragma unroll
+    for (int b = 0; b < NBUF; ++b) issue_next(b);
     // the residual of each of this wavefront's rows, asked for now: at the end of a row the value is
     // there instead of one more trip to memory behind the last weight load
     // (four named registers and a select chain below: an array indexed by the row counter would live in
@@ -110,11 +117,11 @@ __global__ __launch_bounds__(GEMV_THREADS) void gemv_kernel(const GemvArgs a) {
         rms_finish<GEMV_THREADS, GEMV_NORM_R>(xr, xs, K, a.eps, red);
     } else {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
+        for (int j = 0; j < GEMV_XRAW; ++j) {
             const int c = (threadIdx.x + GEMV_THREADS * j) * 8;
             if (c < K) store8(xs + c, xraw[j]);
         }
-        for (int c = (threadIdx.x + GEMV_THREADS * 4) * 8; c < K; c += GEMV_THREADS * 8) store8(xs + c, load8(a.x + c));
+        for (int c = (threadIdx.x + GEMV_THREADS * GEMV_XRAW) * 8; c < K; c += GEMV_THREADS * 8) store8(xs + c, load8(a.x + c));
     }
     __syncthreads();
 
@@ -161,13 +168,14 @@ __global__ __launch_bounds__(GEMV_THREADS) void gemv_kernel(const GemvArgs a) {
         }
         if (++sp == spr) { sp = 0; ++i; }
     };
-    // two steps per trip: each register buffer is refilled right after it is consumed
-    for (int s = 0; s < steps; s += 2) {
-        consume(0);
-        issue_next(0);
-        if (s + 1 < steps) {
-            consume(1);
-            issue_next(1);
+    // NBUF steps per trip: each register buffer is refilled right after it is consumed
+    for (int s = 0; s < steps; s += NBUF) {
+#pragma unroll
+        for (int b = 0; b < NBUF; ++b) {
+            if (s + b < steps) {
+                consume(b);
+                issue_next(b);
+            }
         }
     }
     if (MODE == GV_LMHEAD) {
@@ -237,8 +245,14 @@ __global__ __launch_bounds__(1024) void argmax_final_kernel(const unsigned long 
 // the norm-fused QKV projection and the 128K-row LM head amortise their
 // per-workgroup prologue over more than one row.
 static int rows_per_wave(int mode, int N, bool norm) {
-    if (mode == GV_LMHEAD) return N >= 32768 ? 3 : 1;
-    if (mode == GV_PLAIN && norm && N >= 6144) return 2;
+#ifndef GEMV_RPW_LM
+#define GEMV_RPW_LM 3
+#endif
+#ifndef GEMV_RPW_QKV
+#define GEMV_RPW_QKV 2
+#endif
+    if (mode == GV_LMHEAD) return N >= 32768 ? GEMV_RPW_LM : 1;
+    if (mode == GV_PLAIN && norm && N >= 6144) return GEMV_RPW_QKV;
     return 1;
 }
 
