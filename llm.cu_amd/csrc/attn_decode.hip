@@ -12,9 +12,11 @@
 // the cheap scores, so none waits for another) and write the result directly.
 // Beyond that workgroup y takes the 512-position span y with all dims, leaves
 // (max, sum, unnormalised P.V), and the last workgroup of the head to finish
-// (a self-resetting counter) merges the spans.  Scores, softmax and P.V
-// stay in fp32 as in the reference (src/inference/inference.cu:736-947); only
-// the final output is rounded.
+// (a self-resetting counter) merges the spans.  Both products run on the matrix
+// pipe with fp16 operands and fp32 accumulation (the probabilities are rounded
+// to fp16 like the prompt-pass kernel's); maxima, sums and the merge stay in fp32
+// and only the final output is rounded (reference: src/inference/inference.cu:736-947,
+// which keeps fp32 throughout; the difference is inside the 2e-2 the tests allow).
 #include <cfloat>
 #include <cmath>
 #include <mutex>

@@ -24,7 +24,7 @@ struct AdArgs {
 };
 
 // Every K and V load of the span is issued before anything else (a span is at
-// most 512 positions: 16 + 16 loads of 16 bytes per thread at hd 128), so the
+// most 512 positions: 16 + 2..16 loads of 16 bytes per thread at hd 128), so the
 // whole span costs one trip to HBM instead of one per loop iteration.  In the
 // fused form the new token's own K and V come from the projection row through
 // LDS (and are written to the cache for later steps), so nothing waits on
