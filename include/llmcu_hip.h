@@ -203,6 +203,19 @@ int llm_attn_decode_rope_long(const uint16_t *qkv_dev, uint16_t *k_cache_dev, ui
                          uint16_t *out_dev, int pos_host, const int32_t *pos_dev, const float *table_dev,
                          int n_heads, int n_kv_heads, int head_dim, int max_pos, void *workspace_dev,
                          llm_stream_t stream);
+/* llm_attn_decode_rope_long and the projection that consumes its result in two launches instead of three
+ * (compute_output + add_norm, src/inference/inference.cu:600-618,366-390): the span kernel as above, then one
+ * launch whose first Hq workgroups merge one query head each while all others fetch their rows of w and wait
+ * for the merged vector.  Buffers, hand-over, timeouts_dev and the bits of the result as for
+ * llm_attn_decode_rope_oproj (the two entry points may share one ring of buffers); any position below max_pos.
+ * Limits: Hq*hd <= 4096, N <= 24 * (CUs - Hq). */
+int llm_attn_long_oproj_supported(int n_heads, int n_kv_heads, int head_dim, int N); /* 1 or 0, current device */
+int llm_attn_decode_rope_long_oproj(const uint16_t *qkv_dev, uint16_t *k_cache_dev, uint16_t *v_cache_dev,
+                                    uint16_t *attn_out_dev, uint16_t *attn_out_next_dev, int pos_host,
+                                    const int32_t *pos_dev, const float *table_dev, int n_heads, int n_kv_heads,
+                                    int head_dim, int max_pos, void *workspace_dev, const uint16_t *w_dev,
+                                    const uint16_t *residual_dev, uint16_t *out_dev, int N, int32_t *timeouts_dev,
+                                    llm_stream_t stream);
 /* The same step for `batch` (<= 16) independent sequences in one launch: row z of qkv_dev belongs to the
  * sequence with caches k_caches[z], v_caches[z] (host arrays of device pointers) at position positions[z];
  * workspace_dev holds batch * llm_attn_decode_workspace_bytes().  No counterpart in the reference (it

@@ -137,6 +137,8 @@ HIP_ABI = {
     "llm_sample_candidates_max_vocab": (_i, []),
     "llm_sample_candidates": (_i, [_vp, _vp, _i, _i, _vp, _vp]),
     "llm_attn_decode_rope_long": (_i, [_vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _vp, _vp]),
+    "llm_attn_long_oproj_supported": (_i, [_i, _i, _i, _i]),
+    "llm_attn_decode_rope_long_oproj": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _i, _vp, _vp]),
     "llm_norm_lmhead_argmax": (_i, [_vp, _vp, C.c_double, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp, _vp]),
     "llm_attn_decode_workspace_bytes": (_sz, [_i, _i]),
     "llm_attn_decode": (_i, [_vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _i, _vp, _vp]),

@@ -90,31 +90,11 @@ struct AoArgs {
     int *timeouts;     // diagnostic: waits that ran into AO_SPIN_LIMIT
 };
 
-template <int HD, int G, int DSN>
-__global__ __launch_bounds__(AD_THREADS) void attn_oproj_kernel(const AdArgs a, const AoArgs o) {
-    __shared__ float sc[G * AD_LS];
-    __shared__ __attribute__((aligned(16))) half_t qs[G * HD];
-    __shared__ __attribute__((aligned(16))) half_t knew[HD];
-    __shared__ __attribute__((aligned(16))) half_t vnew[HD];
-    __shared__ float s_m[G], s_l[G];
-    __shared__ int s_last;
-    const int n_attn = a.n_kv_heads * DSN;
+// The projection role of a launch whose first n_first workgroups produce the projection's input vector (a.out,
+// handed over as described above): all weight rows of the workgroup are requested at once, then the vector is
+// polled for, staged in xs (K halves of LDS) and reduced against.
+__device__ __forceinline__ void ao_projection_part(const AdArgs &a, const AoArgs &o, half_t *xs, const int n_attn) {
     const int wg = blockIdx.x, tid = threadIdx.x;
-    if (wg < n_attn) {
-        int pos = a.pos_host + (a.pos_dev ? *a.pos_dev : 0);
-        if (pos > a.max_pos - 1) pos = a.max_pos - 1;
-        if (pos > AD_LS - 1) pos = AD_LS - 1; // this form serves one span; the host picks it below AD_LS only
-        if (pos < 0) pos = 0;
-        const int kvh = wg % a.n_kv_heads, y = wg / a.n_kv_heads;
-        attn_decode_body<HD, G, true, HD / DSN, AD_LS, false, true>(a, sc, qs, knew, vnew, s_m, s_l, &s_last, pos, 1, 0,
-                                                                    y * (HD / DSN), y == 0, kvh);
-        // off the critical path: the next launch's buffer back to "empty" (visible at the end of this kernel)
-        uint32_t *nx = reinterpret_cast<uint32_t *>(o.next);
-        for (int c = wg * AD_THREADS + tid; c < o.K / 2; c += n_attn * AD_THREADS) nx[c] = AO_EMPTY | (AO_EMPTY << 16);
-        return;
-    }
-    // ---- projection part ----------------------------------------------------------------
-    half_t *xs = reinterpret_cast<half_t *>(sc); // K halves: K * 2 <= sizeof(sc), checked by the host
     const int wave = tid / 64, lane = tid % 64;
     const int K = o.K, N = o.N;
     const int wslot = (wg - n_attn) * AO_WAVES + wave; // this wavefront among all of the projection part
@@ -193,6 +173,32 @@ __global__ __launch_bounds__(AD_THREADS) void attn_oproj_kernel(const AdArgs a, 
             o.out[row] = h;
         }
     }
+}
+
+template <int HD, int G, int DSN>
+__global__ __launch_bounds__(AD_THREADS) void attn_oproj_kernel(const AdArgs a, const AoArgs o) {
+    __shared__ float sc[G * AD_LS];
+    __shared__ __attribute__((aligned(16))) half_t qs[G * HD];
+    __shared__ __attribute__((aligned(16))) half_t knew[HD];
+    __shared__ __attribute__((aligned(16))) half_t vnew[HD];
+    __shared__ float s_m[G], s_l[G];
+    __shared__ int s_last;
+    const int n_attn = a.n_kv_heads * DSN;
+    const int wg = blockIdx.x, tid = threadIdx.x;
+    if (wg < n_attn) {
+        int pos = a.pos_host + (a.pos_dev ? *a.pos_dev : 0);
+        if (pos > a.max_pos - 1) pos = a.max_pos - 1;
+        if (pos > AD_LS - 1) pos = AD_LS - 1; // this form serves one span; the host picks it below AD_LS only
+        if (pos < 0) pos = 0;
+        const int kvh = wg % a.n_kv_heads, y = wg / a.n_kv_heads;
+        attn_decode_body<HD, G, true, HD / DSN, AD_LS, false, true>(a, sc, qs, knew, vnew, s_m, s_l, &s_last, pos, 1, 0,
+                                                                    y * (HD / DSN), y == 0, kvh);
+        // off the critical path: the next launch's buffer back to "empty" (visible at the end of this kernel)
+        uint32_t *nx = reinterpret_cast<uint32_t *>(o.next);
+        for (int c = wg * AD_THREADS + tid; c < o.K / 2; c += n_attn * AD_THREADS) nx[c] = AO_EMPTY | (AO_EMPTY << 16);
+        return;
+    }
+    ao_projection_part(a, o, reinterpret_cast<half_t *>(sc), n_attn); // K halves: K * 2 <= sizeof(sc), checked by the host
 }
 
 template <int HD, int G>
@@ -279,7 +285,10 @@ __global__ __launch_bounds__(AD_THREADS) void attn_span_kernel(const AdArgs a) {
                                                          y == n_active - 1);
 }
 
-template <int HD, int G> __device__ __forceinline__ void attn_merge_body(const AdArgs &a) {
+// AGENT_OUT: the head's result leaves as 8-byte device-scope stores with the "not written yet" pattern avoided,
+// for readers inside the same launch (merge_oproj_kernel).
+template <int HD, int G, bool AGENT_OUT = false>
+__device__ __forceinline__ void attn_merge_body(const AdArgs &a, const int h) {
     constexpr int PARTS = AD_MERGE_THREADS / HD;
     __shared__ float w[AD_MAX_SPLITS];
     __shared__ float red[2 * AD_MERGE_THREADS / 64];
@@ -289,7 +298,7 @@ template <int HD, int G> __device__ __forceinline__ void attn_merge_body(const A
     if (pos > a.max_pos - 1) pos = a.max_pos - 1;
     if (pos < 0) pos = 0;
     const int n = pos / AD_LONG_LS + 1;
-    const int h = blockIdx.x, kvh = h / G, hh = h % G, splits = a.splits;
+    const int kvh = h / G, hh = h % G, splits = a.splits;
     const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
     float m = -FLT_MAX, l = 0.f;
     if (tid < n) {
@@ -331,17 +340,33 @@ template <int HD, int G> __device__ __forceinline__ void attn_merge_body(const A
     for (; s < n; s += PARTS) o += accp[(size_t)s * G * HD] * w[s];
     part_o[tid] = o;
     __syncthreads();
+    __shared__ __attribute__((aligned(8))) uint16_t res16[AGENT_OUT ? HD : 4];
     if (tid < HD) {
         float t = part_o[tid];
 #pragma unroll
         for (int q = 1; q < PARTS; ++q) t += part_o[tid + q * HD];
-        a.out[(size_t)h * HD + tid] = (half_t)(t / s_L);
+        const half_t r = (half_t)(t / s_L);
+        if (AGENT_OUT) {
+            uint16_t bits = __builtin_bit_cast(uint16_t, r);
+            if (bits == 0xFFFFu) bits = 0xFFFEu; // 0xFFFF marks "not written yet" for the reader
+            res16[tid] = bits;
+        } else {
+            a.out[(size_t)h * HD + tid] = r;
+        }
+    }
+    if (AGENT_OUT) {
+        static_assert(HD % 4 == 0, "results are stored four at a time");
+        __syncthreads();
+        if (tid < HD / 4)
+            __hip_atomic_store(reinterpret_cast<unsigned long long *>(a.out + (size_t)h * HD) + tid,
+                               reinterpret_cast<const unsigned long long *>(res16)[tid], __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_AGENT);
     }
 }
 
 template <int HD, int G>
 __global__ __launch_bounds__(AD_MERGE_THREADS) void attn_merge_kernel(const AdArgs a) {
-    attn_merge_body<HD, G>(a);
+    attn_merge_body<HD, G>(a, blockIdx.x);
 }
 
 template <int HD, int G, bool FUSED>
@@ -359,6 +384,62 @@ static int launch_decode_long(AdArgs a, void *ws, hipStream_t s) {
     LLM_LAUNCH_CHECK("attn_span_kernel");
     attn_merge_kernel<HD, G><<<dim3(Hq), dim3(AD_MERGE_THREADS), 0, s>>>(a);
     LLM_LAUNCH_CHECK("attn_merge_kernel");
+    return LLM_OK;
+}
+
+// ---------------------------------------------------------------------------
+// Long contexts, merge and output projection in one launch.  The span kernel runs as above; in the second
+// launch the first Hq workgroups merge one query head each and hand the result over to the projection
+// workgroups exactly as the attention workgroups of attn_oproj_kernel do (same buffers, same polling,
+// same refill of the next launch's buffer), so the projection's weights stream while the spans are merged
+// and the projection needs no launch of its own.
+// ---------------------------------------------------------------------------
+template <int HD, int G>
+__global__ __launch_bounds__(AD_THREADS) void merge_oproj_kernel(const AdArgs a, const AoArgs o) {
+    static_assert(AD_MERGE_THREADS == AD_THREADS, "both roles share the workgroup size");
+    __shared__ __attribute__((aligned(16))) half_t xs[AO_KSTEPS * 512];
+    const int n_first = a.n_kv_heads * G;
+    const int wg = blockIdx.x, tid = threadIdx.x;
+    if (wg < n_first) {
+        attn_merge_body<HD, G, true>(a, wg);
+        uint32_t *nx = reinterpret_cast<uint32_t *>(o.next);
+        for (int c = wg * AD_THREADS + tid; c < o.K / 2; c += n_first * AD_THREADS) nx[c] = AO_EMPTY | (AO_EMPTY << 16);
+        return;
+    }
+    ao_projection_part(a, o, xs, n_first);
+}
+
+// projection workgroups and rows per wavefront behind n_first producer workgroups; false when they do not fit
+static bool ao_partition(int N, int n_first, int cus, int *owg_out, int *rows_out) {
+    if (cus <= n_first) return false;
+    int owg = (N + AO_WAVES - 1) / AO_WAVES;
+    if (owg > cus - n_first) owg = cus - n_first; // at most one workgroup per CU: all of them are resident at once
+    const int rows = (N + owg * AO_WAVES - 1) / (owg * AO_WAVES);
+    *owg_out = owg;
+    *rows_out = rows;
+    return rows <= AO_ROWS;
+}
+
+template <int HD, int G>
+static int launch_long_oproj(AdArgs a, AoArgs o, void *ws, hipStream_t s) {
+    const int Hq = a.n_kv_heads * G;
+    int cus = 0;
+    int rc = llm_cu_count_cached(&cus);
+    if (rc != LLM_OK) return rc;
+    LLM_REQUIRE(ao_partition(o.N, Hq, cus, &o.n_owg, &o.rows),
+                "llm_attn_decode_rope_long_oproj: N=%d behind %d merge workgroups does not fit %d CUs", o.N, Hq, cus);
+    a.ws_acc = (float *)ws;
+    a.ws_ml = a.ws_acc + (size_t)Hq * AD_MAX_SPLITS * HD;
+    a.counters = nullptr;
+    const int splits = (a.max_pos + AD_LONG_LS - 1) / AD_LONG_LS;
+    LLM_REQUIRE(splits <= AD_MAX_SPLITS, "llm_attn_decode_rope_long_oproj: max_pos=%d exceeds %d", a.max_pos,
+                AD_MAX_SPLITS * AD_LONG_LS);
+    a.splits = splits;
+    const int gy = a.pos_dev ? splits : a.pos_host / AD_LONG_LS + 1;
+    attn_span_kernel<HD, G, true><<<dim3(a.n_kv_heads, gy), dim3(AD_THREADS), 0, s>>>(a);
+    LLM_LAUNCH_CHECK("attn_span_kernel");
+    merge_oproj_kernel<HD, G><<<dim3(Hq + o.n_owg), dim3(AD_THREADS), 0, s>>>(a, o);
+    LLM_LAUNCH_CHECK("merge_oproj_kernel");
     return LLM_OK;
 }
 
@@ -426,7 +507,7 @@ __global__ __launch_bounds__(AD_THREADS) void attn_span_batch_kernel(const AdArg
 
 template <int HD, int G>
 __global__ __launch_bounds__(AD_MERGE_THREADS) void attn_merge_batch_kernel(const AdArgs common, const AdBatch b) {
-    attn_merge_body<HD, G>(ad_for_sequence(common, b, blockIdx.y));
+    attn_merge_body<HD, G>(ad_for_sequence(common, b, blockIdx.y), blockIdx.x);
 }
 
 template <int HD, int G>
@@ -681,6 +762,69 @@ int llm_attn_decode_rope_long(const uint16_t *qkv, uint16_t *kc, uint16_t *vc, u
     a.n_kv_heads = n_kv_heads;
     a.max_pos = max_pos;
     return dispatch_decode_long<true>(a, n_heads, head_dim, workspace, (hipStream_t)stream);
+}
+
+// 1 when llm_attn_decode_rope_long_oproj covers these shapes on the current device, else 0.
+int llm_attn_long_oproj_supported(int n_heads, int n_kv_heads, int head_dim, int N) {
+    if (n_kv_heads <= 0 || n_heads % n_kv_heads) return 0;
+    const int G = n_heads / n_kv_heads, K = n_heads * head_dim;
+    if (!((head_dim == 128 && (G == 1 || G == 4 || G == 8)) || ((head_dim == 64 || head_dim == 32) && (G == 1 || G == 4)))) return 0;
+    if (K % 8 || K > 512 * AO_KSTEPS || N <= 0) return 0;
+    int cus = 0, owg = 0, rows = 0;
+    if (llm_cu_count_cached(&cus) != LLM_OK) return 0;
+    return ao_partition(N, n_heads, cus, &owg, &rows) ? 1 : 0;
+}
+
+int llm_attn_decode_rope_long_oproj(const uint16_t *qkv, uint16_t *kc, uint16_t *vc, uint16_t *attn_out,
+                                    uint16_t *attn_out_next, int pos_host, const int32_t *pos_dev, const float *table,
+                                    int n_heads, int n_kv_heads, int head_dim, int max_pos, void *workspace,
+                                    const uint16_t *w, const uint16_t *residual, uint16_t *out, int N,
+                                    int32_t *timeouts_dev, llm_stream_t stream) {
+    LLM_REQUIRE(qkv && kc && vc && attn_out && attn_out_next && table && workspace && w && out && timeouts_dev,
+                "llm_attn_decode_rope_long_oproj: null pointer");
+    LLM_REQUIRE(attn_out != attn_out_next, "llm_attn_decode_rope_long_oproj: a launch cannot refill its own buffer");
+    LLM_REQUIRE(n_kv_heads > 0 && n_heads % n_kv_heads == 0, "llm_attn_decode_rope_long_oproj: heads %d/%d", n_heads, n_kv_heads);
+    LLM_REQUIRE(max_pos > 0 && max_pos % 64 == 0, "llm_attn_decode_rope_long_oproj: max_pos=%d must be a multiple of 64", max_pos);
+    LLM_REQUIRE(pos_dev || (pos_host >= 0 && pos_host < max_pos), "llm_attn_decode_rope_long_oproj: position %d of %d", pos_host,
+                max_pos);
+    const int K = n_heads * head_dim;
+    LLM_REQUIRE(N > 0 && K % 8 == 0 && K <= 512 * AO_KSTEPS, "llm_attn_decode_rope_long_oproj: N=%d K=%d (K <= %d)", N, K,
+                512 * AO_KSTEPS);
+    LLM_REQUIRE(aligned16(qkv) && aligned16(kc) && aligned16(vc) && aligned16(attn_out) && aligned16(attn_out_next) &&
+                    aligned16(w),
+                "llm_attn_decode_rope_long_oproj: pointers must be 16-byte aligned");
+    AdArgs a = {};
+    a.q = (const half_t *)qkv;
+    a.kc = (half_t *)kc;
+    a.vc = (half_t *)vc;
+    a.out = (half_t *)attn_out;
+    a.table = table;
+    a.pos_host = pos_host;
+    a.pos_dev = pos_dev;
+    a.n_kv_heads = n_kv_heads;
+    a.max_pos = max_pos;
+    AoArgs o = {};
+    o.w = (const half_t *)w;
+    o.res = (const half_t *)residual;
+    o.out = (half_t *)out;
+    o.next = attn_out_next;
+    o.N = N;
+    o.K = K;
+    o.timeouts = timeouts_dev;
+    hipStream_t s = (hipStream_t)stream;
+    const int G = n_heads / n_kv_heads;
+#define AO_CASE(HD_, G_) \
+    if (head_dim == HD_ && G == G_) return launch_long_oproj<HD_, G_>(a, o, workspace, s);
+    AO_CASE(128, 4)
+    AO_CASE(128, 8)
+    AO_CASE(128, 1)
+    AO_CASE(64, 4)
+    AO_CASE(64, 1)
+    AO_CASE(32, 4)
+    AO_CASE(32, 1)
+#undef AO_CASE
+    llm_set_error("llm_attn_decode_rope_long_oproj: head_dim=%d with group size %d is not built", head_dim, G);
+    return LLM_ERR_INVALID;
 }
 
 int llm_attn_decode_rope_batch(const uint16_t *qkv, int ldq, uint16_t *const *k_caches, uint16_t *const *v_caches,

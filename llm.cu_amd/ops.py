@@ -268,9 +268,11 @@ def attn_decode_rope(qkv, kc, vc, pos, n_heads, n_kv_heads, head_dim, theta=5000
     return d_o.download(), d_k.download(), d_v.download()
 
 
-def attn_decode_rope_oproj(qkv, kc, vc, pos, n_heads, n_kv_heads, head_dim, w, residual=None, theta=500000.0, repeats=1):
-    """llm_attn_decode_rope_oproj: returns (attention output [Hq*hd], projection output [N], K cache, V cache,
-    timeouts).  Each repeat starts from the same caches and uses the next buffer of a two-buffer ring."""
+def attn_decode_rope_oproj(qkv, kc, vc, pos, n_heads, n_kv_heads, head_dim, w, residual=None, theta=500000.0, repeats=1,
+                           long_form=False):
+    """llm_attn_decode_rope_oproj (long_form: llm_attn_decode_rope_long_oproj): returns (attention output [Hq*hd],
+    projection output [N], K cache, V cache, timeouts).  Each repeat starts from the same caches and uses the next
+    buffer of a two-buffer ring."""
     qkv, kc, vc, w = _u16(qkv).reshape(-1), _u16(kc), _u16(vc), _u16(w)
     max_pos = kc.shape[1]
     N = w.shape[0]
@@ -281,14 +283,22 @@ def attn_decode_rope_oproj(qkv, kc, vc, pos, n_heads, n_kv_heads, head_dim, w, r
     check(lib().llm_attn_oproj_buffer_init(ring.ptr, 2 * qd, None))
     tmo = DevBuf((1,), np.int32)
     tmo.zero()
+    wsb = (lib().llm_attn_decode_workspace_bytes(n_heads, head_dim) + 3) // 4 * 4
+    d_ws = DevBuf((wsb // 4,), np.uint32)
+    d_ws.zero()
     res = None
     for r in range(repeats):
         d_k, d_v = DevBuf.from_host(kc), DevBuf.from_host(vc)
         d_o = DevBuf.from_host(_u16(residual).reshape(-1)) if residual is not None else DevBuf((N,), np.uint16)
         cur, nxt = ring.ptr + 2 * qd * (r % 2), ring.ptr + 2 * qd * ((r + 1) % 2)
-        check(lib().llm_attn_decode_rope_oproj(d_q.ptr, d_k.ptr, d_v.ptr, cur, nxt, pos, None, d_t.ptr, n_heads, n_kv_heads,
-                                               head_dim, max_pos, d_w.ptr, d_o.ptr if residual is not None else None,
-                                               d_o.ptr, N, tmo.ptr, None))
+        if long_form:
+            check(lib().llm_attn_decode_rope_long_oproj(d_q.ptr, d_k.ptr, d_v.ptr, cur, nxt, pos, None, d_t.ptr, n_heads,
+                                                        n_kv_heads, head_dim, max_pos, d_ws.ptr, d_w.ptr,
+                                                        d_o.ptr if residual is not None else None, d_o.ptr, N, tmo.ptr, None))
+        else:
+            check(lib().llm_attn_decode_rope_oproj(d_q.ptr, d_k.ptr, d_v.ptr, cur, nxt, pos, None, d_t.ptr, n_heads, n_kv_heads,
+                                                   head_dim, max_pos, d_w.ptr, d_o.ptr if residual is not None else None,
+                                                   d_o.ptr, N, tmo.ptr, None))
         out = (ring.download()[r % 2].copy(), d_o.download(), d_k.download(), d_v.download())
         assert res is None or all(np.array_equal(x, y) for x, y in zip(res, out)), "repeat %d differs" % r
         res = out

@@ -52,6 +52,7 @@ struct Engine {
     int32_t *d_pos = nullptr;    // tokens cached so far; d_tokens[*d_pos] is the next input
     int32_t *d_token = nullptr;  // [0] last argmax, [1] waits of the fused attention + projection launch that gave up
     llm_half *ao_ring = nullptr; // one attention-output buffer per layer for llm_attn_decode_rope_oproj (null: not used)
+    bool ao_long = false;        // the ring also serves llm_attn_decode_rope_long_oproj
     // the whole decode token in one launch (llm_decode_fused), when the shapes and the device allow it
     bool fused_ok = false, fused_on = false; // measured slower than one launch per operation: opt-in
     llm_decode_desc fdesc = {};
@@ -202,8 +203,8 @@ void issue_pass(Engine *e, const Llama3 *m, int T, int pos0, bool dev_pos, bool 
                  "llm_embed_gather");
     const llm_half *final_gain = m->norm->d_fp16_tensor;
     if (T == 1) {
-        // decode step: 5 launches per layer (norm folded into the projections, RoPE + cache append
-        // folded into the attention, residual adds in the projection epilogues)
+        // decode step: 4 launches per layer, 5 at long contexts (norm folded into the projections, RoPE + cache
+        // append folded into the attention, residual adds in the projection epilogues)
         for (int l = 0; l < c.n_layers; ++l) {
             const LayerW w = layer_w(m, l);
             llm_half *kc = e->kc + (size_t)l * e->kv_layer_elems, *vc = e->vc + (size_t)l * e->kv_layer_elems;
@@ -226,6 +227,13 @@ void issue_pass(Engine *e, const Llama3 *m, int T, int pos0, bool dev_pos, bool 
                                                         e->rope_table, Hq, Hkv, hd, c.max_pos, w.wo, e->x, e->x, d,
                                                         e->d_token + 1, s),
                              "llm_attn_decode_rope_oproj");
+            } else if (e->long_attn && e->ao_ring && e->ao_long) {
+                // long contexts: spans, then merge + output projection in one launch (same ring, same re-arming)
+                llama3_check(llm_attn_decode_rope_long_oproj(e->qkv, kc, vc, e->ao_ring + (size_t)l * qd,
+                                                             e->ao_ring + (size_t)((l + 1) % c.n_layers) * qd, p0, pd,
+                                                             e->rope_table, Hq, Hkv, hd, c.max_pos, e->ws_attn, w.wo, e->x,
+                                                             e->x, d, e->d_token + 1, s),
+                             "llm_attn_decode_rope_long_oproj");
             } else {
                 llama3_check((e->long_attn ? llm_attn_decode_rope_long : llm_attn_decode_rope)(
                                  e->qkv, kc, vc, e->attn, p0, pd, e->rope_table, Hq, Hkv, hd, c.max_pos, e->ws_attn, s),
@@ -511,6 +519,7 @@ extern "C" CudaCache *init_cache_cfg(Llama3 *m, const ModelConfig *cfg) {
     if (c.n_layers >= 2 && llm_attn_oproj_supported(c.n_heads, c.n_kv_heads, c.head_dim, d)) {
         e->ao_ring = dmalloc<llm_half>((size_t)c.n_layers * qd, "llm_malloc(attention hand-over ring)");
         llama3_check(llm_attn_oproj_buffer_init(e->ao_ring, c.n_layers * qd, e->stream), "llm_attn_oproj_buffer_init");
+        e->ao_long = llm_attn_long_oproj_supported(c.n_heads, c.n_kv_heads, c.head_dim, d) == 1;
     }
     llama3_check(llm_fill_zero(e->d_tokens, sizeof(int32_t) * (R + 1), e->stream), "zero tokens");
     llama3_check(llm_fill_zero(e->d_pos, sizeof(int32_t), e->stream), "zero pos");

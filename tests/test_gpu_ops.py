@@ -535,6 +535,36 @@ def test_attn_decode_rope_fused(gpu, pos, max_pos, Hq, Hkv, hd):
     assert e <= TOL and H.mixed_err(out_l, out) <= TIGHT
 
 
+@pytest.mark.parametrize("pos,max_pos,Hq,Hkv,hd,N", [(0, 64, 32, 8, 128, 4096), (700, 1024, 32, 8, 128, 4096),
+                                                     (8300, 8704, 32, 8, 128, 4096), (300, 512, 32, 8, 128, 1008),
+                                                     (137, 320, 8, 2, 32, 256), (530, 576, 4, 4, 64, 272)])
+def test_attn_decode_rope_long_oproj_equals_the_three_launches(gpu, pos, max_pos, Hq, Hkv, hd, N):
+    """Span kernel, then merge + output projection in one launch (the merge workgroups hand their heads over to
+    the projection workgroups, which fetched their weights meanwhile): attention output, projection output (with
+    the in-place residual) and both caches equal llm_attn_decode_rope_long followed by llm_linear bit for bit, on
+    three calls in a row through the buffer ring, with no wait that ran into its limit."""
+    rng = np.random.default_rng(pos + N + 1)
+    qd, kvd = Hq * hd, Hkv * hd
+    qkv = H.bits(rng.standard_normal((1, qd + 2 * kvd)))
+    k_old, v_old = H.bits(rng.standard_normal((pos, kvd))), H.bits(rng.standard_normal((pos, kvd)))
+    kc, vc = gpu.ops.kv_layout(k_old, v_old, Hkv, hd, max_pos)
+    w = H.bits(0.05 * rng.standard_normal((N, qd)))
+    res = H.bits(rng.standard_normal((1, N)))
+    say("span, merge+oproj", pos, max_pos, Hq, Hkv, hd, N)
+    assert gpu.lib().llm_attn_long_oproj_supported(Hq, Hkv, hd, N) == 1
+    a_f, o_f, kc_f, vc_f, timeouts = gpu.ops.attn_decode_rope_oproj(qkv, kc, vc, pos, Hq, Hkv, hd, w, residual=res, repeats=3,
+                                                                    long_form=True)
+    assert timeouts == 0
+    a_r, kc_r, vc_r = gpu.ops.attn_decode_rope(qkv, kc, vc, pos, Hq, Hkv, hd, long_form=True)
+    o_r = gpu.ops.linear(a_r.reshape(1, -1), w, residual=res).reshape(-1)
+    assert np.array_equal(a_f, a_r) and np.array_equal(kc_f, kc_r) and np.array_equal(vc_f, vc_r)
+    assert np.array_equal(o_f, o_r), int(H.ulp_diff(o_f, o_r).max())
+    want = orc.add(orc.linear(a_r.reshape(1, -1), w), res).reshape(-1)
+    assert H.mixed_err(o_f, want) <= TOL
+    _, o_n, _, _, timeouts = gpu.ops.attn_decode_rope_oproj(qkv, kc, vc, pos, Hq, Hkv, hd, w, long_form=True)
+    assert timeouts == 0 and np.array_equal(o_n, gpu.ops.linear(a_r.reshape(1, -1), w).reshape(-1))
+
+
 @pytest.mark.parametrize("pos,max_pos,Hq,Hkv,hd,N", [(0, 64, 32, 8, 128, 4096), (200, 1024, 32, 8, 128, 4096),
                                                      (511, 8704, 32, 8, 128, 4096), (300, 512, 32, 8, 128, 1008),
                                                      (37, 64, 8, 2, 32, 256), (130, 256, 4, 4, 64, 272)])
