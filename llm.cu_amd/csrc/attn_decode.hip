@@ -264,7 +264,8 @@ static int dispatch_decode(AdArgs a, int n_heads, int head_dim, void *ws, hipStr
 // query head, combines them.  No fence, counter or last-workgroup tail: beyond a few spans that tail
 // costs more than the second launch.
 // ---------------------------------------------------------------------------
-#define AD_LONG_LS 256
+#define AD_LONG_LS 256      // shortest span of the long form (ad_long_span_len)
+#define AD_LONG_LS_MAX 512  // longest
 #define AD_MERGE_THREADS 512
 
 template <int HD, int G, bool FUSED>
@@ -278,11 +279,12 @@ __global__ __launch_bounds__(AD_THREADS) void attn_span_kernel(const AdArgs a) {
     int pos = a.pos_host + (a.pos_dev ? *a.pos_dev : 0);
     if (pos > a.max_pos - 1) pos = a.max_pos - 1;
     if (pos < 0) pos = 0;
-    const int n_active = pos / AD_LONG_LS + 1;
+    const int span_len = ad_long_span_len(pos + 1, a.span_target);
+    const int n_active = ad_long_spans(pos + 1, a.span_target);
     const int y = blockIdx.y;
     if (y >= n_active) return;
-    attn_decode_body<HD, G, FUSED, HD, AD_LONG_LS, true>(a, sc, qs, knew, vnew, s_m, s_l, &s_last, pos, n_active, y, 0,
-                                                         y == n_active - 1);
+    attn_decode_body<HD, G, FUSED, HD, AD_LONG_LS_MAX, true>(a, sc, qs, knew, vnew, s_m, s_l, &s_last, pos, n_active, y, 0,
+                                                             y == n_active - 1, -1, nullptr, nullptr, span_len);
 }
 
 // AGENT_OUT: the head's result leaves as 8-byte device-scope stores with the "not written yet" pattern avoided,
@@ -297,7 +299,7 @@ __device__ __forceinline__ void attn_merge_body(const AdArgs &a, const int h) {
     int pos = a.pos_host + (a.pos_dev ? *a.pos_dev : 0);
     if (pos > a.max_pos - 1) pos = a.max_pos - 1;
     if (pos < 0) pos = 0;
-    const int n = pos / AD_LONG_LS + 1;
+    const int n = ad_long_spans(pos + 1, a.span_target);
     const int kvh = h / G, hh = h % G, splits = a.splits;
     const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
     float m = -FLT_MAX, l = 0.f;
@@ -369,17 +371,35 @@ __global__ __launch_bounds__(AD_MERGE_THREADS) void attn_merge_kernel(const AdAr
     attn_merge_body<HD, G>(a, blockIdx.x);
 }
 
+// Long form on the host: the span target of this device (a.span_target) and the second grid dimension of the span
+// kernel (the spans in use when the position is known here, else the most that any position below max_pos needs).
+static int ad_long_setup(AdArgs &a, int *gy) {
+    int cus = 0;
+    int rc = llm_cu_count_cached(&cus);
+    if (rc != LLM_OK) return rc;
+    a.span_target = cus / a.n_kv_heads > 0 ? cus / a.n_kv_heads : 1;
+    const int splits = (a.max_pos + AD_LONG_LS - 1) / AD_LONG_LS; // spans of the workspace layout: never fewer than in use
+    LLM_REQUIRE(splits <= AD_MAX_SPLITS, "decode attention: max_pos=%d exceeds %d", a.max_pos, AD_MAX_SPLITS * AD_LONG_LS);
+    a.splits = splits;
+    if (a.pos_dev) {
+        const int knee = a.span_target * AD_LONG_LS < a.max_pos ? a.span_target * AD_LONG_LS : a.max_pos;
+        const int m1 = ad_long_spans(knee, a.span_target), m2 = ad_long_spans(a.max_pos, a.span_target);
+        *gy = m1 > m2 ? m1 : m2;
+    } else {
+        *gy = ad_long_spans(a.pos_host + 1, a.span_target);
+    }
+    return LLM_OK;
+}
+
 template <int HD, int G, bool FUSED>
 static int launch_decode_long(AdArgs a, void *ws, hipStream_t s) {
     const int Hq = a.n_kv_heads * G;
     a.ws_acc = (float *)ws;
     a.ws_ml = a.ws_acc + (size_t)Hq * AD_MAX_SPLITS * HD;
     a.counters = nullptr;
-    const int splits = (a.max_pos + AD_LONG_LS - 1) / AD_LONG_LS;
-    LLM_REQUIRE(splits <= AD_MAX_SPLITS, "llm_attn_decode: max_pos=%d exceeds %d", a.max_pos, AD_MAX_SPLITS * AD_LONG_LS);
-    a.splits = splits;
-    // with the position known on the host only the spans in use are launched
-    const int gy = a.pos_dev ? splits : a.pos_host / AD_LONG_LS + 1;
+    int gy = 0;
+    int rc = ad_long_setup(a, &gy);
+    if (rc != LLM_OK) return rc;
     attn_span_kernel<HD, G, FUSED><<<dim3(a.n_kv_heads, gy), dim3(AD_THREADS), 0, s>>>(a);
     LLM_LAUNCH_CHECK("attn_span_kernel");
     attn_merge_kernel<HD, G><<<dim3(Hq), dim3(AD_MERGE_THREADS), 0, s>>>(a);
@@ -431,11 +451,9 @@ static int launch_long_oproj(AdArgs a, AoArgs o, void *ws, hipStream_t s) {
     a.ws_acc = (float *)ws;
     a.ws_ml = a.ws_acc + (size_t)Hq * AD_MAX_SPLITS * HD;
     a.counters = nullptr;
-    const int splits = (a.max_pos + AD_LONG_LS - 1) / AD_LONG_LS;
-    LLM_REQUIRE(splits <= AD_MAX_SPLITS, "llm_attn_decode_rope_long_oproj: max_pos=%d exceeds %d", a.max_pos,
-                AD_MAX_SPLITS * AD_LONG_LS);
-    a.splits = splits;
-    const int gy = a.pos_dev ? splits : a.pos_host / AD_LONG_LS + 1;
+    int gy = 0;
+    rc = ad_long_setup(a, &gy);
+    if (rc != LLM_OK) return rc;
     attn_span_kernel<HD, G, true><<<dim3(a.n_kv_heads, gy), dim3(AD_THREADS), 0, s>>>(a);
     LLM_LAUNCH_CHECK("attn_span_kernel");
     merge_oproj_kernel<HD, G><<<dim3(Hq + o.n_owg), dim3(AD_THREADS), 0, s>>>(a, o);
@@ -498,11 +516,12 @@ __global__ __launch_bounds__(AD_THREADS) void attn_span_batch_kernel(const AdArg
     __shared__ float s_m[G], s_l[G];
     __shared__ int s_last;
     const AdArgs a = ad_for_sequence(common, b, blockIdx.z);
-    const int n_active = a.pos_host / AD_LONG_LS + 1;
+    const int span_len = ad_long_span_len(a.pos_host + 1, a.span_target);
+    const int n_active = ad_long_spans(a.pos_host + 1, a.span_target);
     const int y = blockIdx.y;
     if (y >= n_active) return;
-    attn_decode_body<HD, G, true, HD, AD_LONG_LS, true>(a, sc, qs, knew, vnew, s_m, s_l, &s_last, a.pos_host, n_active,
-                                                        y, 0, y == n_active - 1);
+    attn_decode_body<HD, G, true, HD, AD_LONG_LS_MAX, true>(a, sc, qs, knew, vnew, s_m, s_l, &s_last, a.pos_host, n_active,
+                                                            y, 0, y == n_active - 1, -1, nullptr, nullptr, span_len);
 }
 
 template <int HD, int G>
@@ -524,10 +543,17 @@ static int launch_decode_batch(AdArgs a, const AdBatch &b, int B, void *ws, hipS
     }
     a.ws_acc = (float *)ws;
     a.ws_ml = a.ws_acc + (size_t)Hq * AD_MAX_SPLITS * HD;
-    const int splits = (a.max_pos + AD_LONG_LS - 1) / AD_LONG_LS;
-    LLM_REQUIRE(splits <= AD_MAX_SPLITS, "llm_attn_decode_batch: max_pos=%d exceeds %d", a.max_pos, AD_MAX_SPLITS * AD_LONG_LS);
-    a.splits = splits;
-    attn_span_batch_kernel<HD, G><<<dim3(a.n_kv_heads, max_pos_used / AD_LONG_LS + 1, B), dim3(AD_THREADS), 0, s>>>(a, b);
+    int gy = 0;
+    a.pos_dev = nullptr;
+    a.pos_host = 0;
+    int rc = ad_long_setup(a, &gy);
+    if (rc != LLM_OK) return rc;
+    gy = 1;
+    for (int z = 0; z < B; ++z) { // the sequence with the most spans sizes the grid (not always the longest one)
+        const int n = ad_long_spans(b.pos[z] + 1, a.span_target);
+        gy = n > gy ? n : gy;
+    }
+    attn_span_batch_kernel<HD, G><<<dim3(a.n_kv_heads, gy, B), dim3(AD_THREADS), 0, s>>>(a, b);
     LLM_LAUNCH_CHECK("attn_span_batch_kernel");
     attn_merge_batch_kernel<HD, G><<<dim3(Hq, B), dim3(AD_MERGE_THREADS), 0, s>>>(a, b);
     LLM_LAUNCH_CHECK("attn_merge_batch_kernel");

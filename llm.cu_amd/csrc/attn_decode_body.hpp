@@ -19,9 +19,24 @@ struct AdArgs {
     int pos_host;
     const int32_t *pos_dev; // position of the new token = pos_host + *pos_dev; ctx = position + 1
     int n_kv_heads, max_pos, splits;
+    int span_target;   // long form: spans per kv head that fill the device once (CUs / kv heads, at least 1)
     float *ws_acc, *ws_ml;
     int *counters;
 };
+
+// Long form: length of a span and number of spans for a context of ctx positions.  256 positions while that
+// needs no more than `target` spans per kv head (one workgroup per CU); beyond that the spans grow, in steps of
+// 32 positions (a wavefront's block) up to 512, so that the span workgroups still run side by side instead of
+// leaving a few for a second round; beyond target * 512 positions the spans stay at 512.
+__host__ __device__ inline int ad_long_span_len(int ctx, int target) {
+    if (target < 1) target = 1;
+    int per = ((ctx + target - 1) / target + 31) / 32 * 32;
+    return per < 256 ? 256 : per > 512 ? 512 : per;
+}
+__host__ __device__ inline int ad_long_spans(int ctx, int target) {
+    const int len = ad_long_span_len(ctx, target);
+    return (ctx + len - 1) / len;
+}
 
 // Every K and V load of the span is issued before anything else (a span is at
 // most 512 positions: 16 + 2..16 loads of 16 bytes per thread at hd 128), so the
@@ -70,7 +85,8 @@ template <int HD, int G, bool FUSED, int NDIM, int LS, bool TWOPASS, bool AGENT_
 __device__ __forceinline__ void attn_decode_span(const AdArgs &a, half_t *qs, half_t *knew, half_t *vnew,
                                                  half_t *kst_all, float *ow_all, float *ml_all, const int pos,
                                                  const int n_active, const int split, const int d_begin,
-                                                 const bool appender, const int kvh, half_t *qkv_l, int *timeouts) {
+                                                 const bool appender, const int kvh, half_t *qkv_l, int *timeouts,
+                                                 const int span_len) {
     constexpr int LPP = HD / 8;   // lanes per K row
     constexpr int PPW = 64 / LPP; // K rows per load instruction of a wavefront
     constexpr int NPB = 32 / PPW; // load instructions per block
@@ -85,8 +101,8 @@ __device__ __forceinline__ void attn_decode_span(const AdArgs &a, half_t *qs, ha
     const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
     const int max_pos = a.max_pos;
     const int ctx = pos + 1;
-    const int s0 = split * LS;
-    const int len = ctx - s0 < LS ? ctx - s0 : LS;
+    const int s0 = split * span_len; // span_len <= LS
+    const int len = ctx - s0 < span_len ? ctx - s0 : span_len;
     half_t *kbase = a.kc + (size_t)kvh * max_pos * HD;
     half_t *vrow0 = a.vc + (size_t)kvh * HD * max_pos;
     const int lpos = pos - s0; // the new token inside this span (last span only)
@@ -125,24 +141,28 @@ __device__ __forceinline__ void attn_decode_span(const AdArgs &a, half_t *qs, ha
     if (!FUSED && tid * 8 < G * HD) q_r = load8(a.q + (size_t)kvh * G * HD + tid * 8);
 
     // ---- 1. every K and V load of the wavefront's blocks -----------------------------------
+    // (The span kernels of the long form, whose spans may end anywhere between 256 and 512 positions, skip a
+    // second block that lies beyond the span altogether: there the uncounted waits cost less than the loads.)
     half8_t kreg[NB][NPB];
 #pragma unroll
     for (int c = 0; c < NB; ++c) {
+        const bool on = !TWOPASS || c == 0 || 256 * c + blk0 < len; // wave-uniform
 #pragma unroll
         for (int q = 0; q < NPB; ++q) {
             const int j = 256 * c + blk0 + q * PPW + prow;
             const int jc = j < len ? j : len - 1;
-            kreg[c][q] = load8(kbase + (size_t)(s0 + jc) * HD + sub * 8);
+            kreg[c][q] = on ? load8(kbase + (size_t)(s0 + jc) * HD + sub * 8) : half8_t{0, 0, 0, 0, 0, 0, 0, 0};
         }
     }
     half8_t vreg[NB][NT]; // lane (mg, mn): dim 16 t + mn, positions 8 mg .. + 7 of the block
 #pragma unroll
     for (int c = 0; c < NB; ++c) {
+        const bool on = !TWOPASS || c == 0 || 256 * c + blk0 < len;
         const int j = 256 * c + blk0 + 8 * mg;
         const int jc = j < len ? j : ((len - 1) & ~7);
 #pragma unroll
         for (int t = 0; t < NT; ++t)
-            vreg[c][t] = load8(vrow0 + (size_t)(d_begin + 16 * t + mn) * max_pos + s0 + jc);
+            vreg[c][t] = on ? load8(vrow0 + (size_t)(d_begin + 16 * t + mn) * max_pos + s0 + jc) : half8_t{0, 0, 0, 0, 0, 0, 0, 0};
     }
 
     // ---- 2. queries into LDS; fused: rotate them and the new K, append K/V ---------
@@ -354,20 +374,21 @@ __device__ __forceinline__ void attn_decode_body(const AdArgs &a, float *sc, hal
                                                  float *s_m, float *s_l, int *s_last, const int pos,
                                                  const int n_active, const int split, const int d_begin,
                                                  const bool appender, const int kvh_arg = -1, half_t *qkv_l = nullptr,
-                                                 int *timeouts = nullptr) {
+                                                 int *timeouts = nullptr, const int span_len_arg = 0) {
     static_assert(LS == 256 || LS == 512, "span length");
+    const int span_len = span_len_arg > 0 ? span_len_arg : LS; // positions per span (a multiple of 8, at most LS)
     half_t *kst_all = ad_lds_kst<HD>();  // K blocks, one slice per wavefront
     float *ow_all = ad_lds_ow<NDIM, G>();  // unnormalised P.V per wavefront
     float *ml_all = ad_lds_ml<G>();      // (max, sum) per wavefront and head
     const int kvh = kvh_arg >= 0 ? kvh_arg : (int)blockIdx.x, splits = a.splits;
     const int tid = threadIdx.x;
     // one or two blocks per wavefront, each form with its own fixed number of loads in flight
-    if (LS == 512 && pos + 1 - split * LS > 256)
+    if (LS == 512 && pos + 1 - split * span_len > 256 && span_len > 256)
         attn_decode_span<HD, G, FUSED, NDIM, LS, TWOPASS, AGENT_OUT, POLL_IN, LS / 256>(
-            a, qs, knew, vnew, kst_all, ow_all, ml_all, pos, n_active, split, d_begin, appender, kvh, qkv_l, timeouts);
+            a, qs, knew, vnew, kst_all, ow_all, ml_all, pos, n_active, split, d_begin, appender, kvh, qkv_l, timeouts, span_len);
     else
         attn_decode_span<HD, G, FUSED, NDIM, LS, TWOPASS, AGENT_OUT, POLL_IN, 1>(
-            a, qs, knew, vnew, kst_all, ow_all, ml_all, pos, n_active, split, d_begin, appender, kvh, qkv_l, timeouts);
+            a, qs, knew, vnew, kst_all, ow_all, ml_all, pos, n_active, split, d_begin, appender, kvh, qkv_l, timeouts, span_len);
     if (n_active == 1 && !TWOPASS) return;
     if (TWOPASS) return; // attn_merge_kernel combines the spans
 
