@@ -503,7 +503,13 @@ def test_norm_lmhead_argmax_equals_unfused(gpu):
 @pytest.mark.parametrize("pos,max_pos,Hq,Hkv,hd", [(0, 64, 8, 2, 32), (37, 64, 8, 2, 32), (0, 2048, 32, 8, 128),
                                                    (300, 2048, 32, 8, 128), (511, 2048, 32, 8, 128),
                                                    (512, 2048, 32, 8, 128), (1500, 2048, 32, 8, 128),
-                                                   (8447, 8704, 32, 8, 128)])
+                                                   (8447, 8704, 32, 8, 128),
+                                                   # long form around the points where its span length changes on a
+                                                   # 256-CU device (spans of 256 up to 8192 positions, then growing
+                                                   # in steps of 32 up to 512; beyond 16384 more than 32 spans)
+                                                   (8191, 16640, 32, 8, 128), (8192, 16640, 32, 8, 128),
+                                                   (12287, 16640, 32, 8, 128), (16383, 16640, 32, 8, 128),
+                                                   (16600, 16640, 32, 8, 128)])
 def test_attn_decode_rope_fused(gpu, pos, max_pos, Hq, Hkv, hd):
     """RoPE + cache append + attention in one launch == llm_rope_kv_append then llm_attn_decode, and == oracle."""
     rng = np.random.default_rng(pos + hd)
