@@ -411,6 +411,17 @@ def test_errors_are_reported_not_swallowed(gpu):
     assert b"null" in L.llm_last_error()
     buf = gpu.capi.DevBuf((64,), np.uint16)
     assert L.llm_linear(buf.ptr, 60, buf.ptr, None, 0, buf.ptr, 64, 1, 64, 60, None) == gpu.capi.LLM_ERR_INVALID
+    # the launches that hand a vector over inside one kernel: a buffer cannot be its own successor, the
+    # position must exist, unsupported shapes say so (nothing is launched in any of these calls)
+    big = gpu.capi.DevBuf((1 << 16,), np.uint16)
+    p = big.ptr
+    for fn, extra in ((L.llm_attn_decode_rope_oproj, ()), (L.llm_attn_decode_rope_long_oproj, (p,))):
+        args = lambda out, nxt, pos, hq: (p, p, p, out, nxt, pos, None, p, hq, 2, 32, 64) + extra + (p, None, p, 64, p, None)
+        assert fn(*args(p, p, 3, 8)) == gpu.capi.LLM_ERR_INVALID and b"refill" in L.llm_last_error()
+        assert fn(*args(p, p + 4096, 64, 8)) == gpu.capi.LLM_ERR_INVALID and b"position" in L.llm_last_error()
+        assert fn(*args(p, p + 4096, 3, 6)) == gpu.capi.LLM_ERR_INVALID and b"not built" in L.llm_last_error()
+    assert L.llm_attn_long_oproj_supported(32, 8, 128, 4096) == 1 and L.llm_attn_long_oproj_supported(32, 8, 128, 1 << 20) == 0
+    assert L.llm_attn_long_oproj_supported(6, 2, 32, 64) == 0 and L.llm_attn_oproj_supported(6, 2, 32, 64) == 0
 
 
 def test_llama3_8b_two_layers_parity(gpu):
