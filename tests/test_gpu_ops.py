@@ -376,6 +376,21 @@ def test_attn_decode_llama3_8b_heads(gpu, ctx, max_pos):
     assert e <= TOL
 
 
+@pytest.mark.parametrize("ctx,Hq,Hkv,hd", [(300, 16, 2, 128), (700, 16, 2, 128), (400, 4, 4, 128), (1500, 4, 4, 128),
+                                          (260, 8, 2, 64), (900, 8, 2, 64), (513, 2, 2, 32), (40, 4, 4, 64)])
+def test_attn_decode_other_head_shapes(gpu, ctx, Hq, Hkv, hd):
+    """llm_attn_decode (queries already rotated, token already in the cache) for the group sizes and head sizes
+    besides the 8B one: one span, two blocks per wavefront, several spans merged by the last workgroup."""
+    q, k, v = _attn_inputs(ctx + Hq, ctx, Hq, Hkv, hd)
+    kc, vc = gpu.ops.kv_layout(k, v, Hkv, hd, 2048)
+    say("attn decode", ctx, Hq, Hkv, hd)
+    got = gpu.ops.attn_decode(q[-1], kc, vc, ctx, Hq, Hkv, hd, repeats=2)
+    want = orc.attention(q[-1:], k, v, ctx - 1, Hq, Hkv, hd).reshape(-1)
+    e = H.mixed_err(got, want)
+    say("  err", e)
+    assert e <= TOL
+
+
 def test_attn_decode_small_heads_and_gqa_map(gpu):
     Hq, Hkv, hd, ctx = 8, 2, 32, 20
     q, k, v = _attn_inputs(3, ctx, Hq, Hkv, hd)
@@ -509,7 +524,14 @@ def test_norm_lmhead_argmax_equals_unfused(gpu):
                                                    # in steps of 32 up to 512; beyond 16384 more than 32 spans)
                                                    (8191, 16640, 32, 8, 128), (8192, 16640, 32, 8, 128),
                                                    (12287, 16640, 32, 8, 128), (16383, 16640, 32, 8, 128),
-                                                   (16600, 16640, 32, 8, 128)])
+                                                   (16600, 16640, 32, 8, 128),
+                                                   # the other head shapes the kernels are built for: groups of 8 and
+                                                   # of 1 at head size 128, head sizes 64 and 32, one and two blocks
+                                                   # per wavefront, short and long form
+                                                   (100, 1024, 16, 2, 128), (400, 1024, 16, 2, 128), (900, 1024, 16, 2, 128),
+                                                   (300, 1024, 4, 4, 128), (700, 1024, 4, 4, 128),
+                                                   (450, 1024, 8, 2, 64), (600, 1024, 8, 2, 64), (77, 1024, 4, 4, 64),
+                                                   (500, 1024, 2, 2, 32), (1000, 1024, 2, 2, 32)])
 def test_attn_decode_rope_fused(gpu, pos, max_pos, Hq, Hkv, hd):
     """RoPE + cache append + attention in one launch == llm_rope_kv_append then llm_attn_decode, and == oracle."""
     rng = np.random.default_rng(pos + hd)
@@ -543,7 +565,9 @@ def test_attn_decode_rope_fused(gpu, pos, max_pos, Hq, Hkv, hd):
 
 @pytest.mark.parametrize("pos,max_pos,Hq,Hkv,hd,N", [(0, 64, 32, 8, 128, 4096), (700, 1024, 32, 8, 128, 4096),
                                                      (8300, 8704, 32, 8, 128, 4096), (300, 512, 32, 8, 128, 1008),
-                                                     (137, 320, 8, 2, 32, 256), (530, 576, 4, 4, 64, 272)])
+                                                     (137, 320, 8, 2, 32, 256), (530, 576, 4, 4, 64, 272),
+                                                     (900, 1024, 16, 2, 128, 2048), (600, 1024, 4, 4, 128, 512),
+                                                     (700, 1024, 8, 2, 64, 512), (1000, 1024, 2, 2, 32, 64)])
 def test_attn_decode_rope_long_oproj_equals_the_three_launches(gpu, pos, max_pos, Hq, Hkv, hd, N):
     """Span kernel, then merge + output projection in one launch (the merge workgroups hand their heads over to
     the projection workgroups, which fetched their weights meanwhile): attention output, projection output (with
@@ -573,7 +597,9 @@ def test_attn_decode_rope_long_oproj_equals_the_three_launches(gpu, pos, max_pos
 
 @pytest.mark.parametrize("pos,max_pos,Hq,Hkv,hd,N", [(0, 64, 32, 8, 128, 4096), (200, 1024, 32, 8, 128, 4096),
                                                      (511, 8704, 32, 8, 128, 4096), (300, 512, 32, 8, 128, 1008),
-                                                     (37, 64, 8, 2, 32, 256), (130, 256, 4, 4, 64, 272)])
+                                                     (37, 64, 8, 2, 32, 256), (130, 256, 4, 4, 64, 272),
+                                                     (333, 512, 16, 2, 128, 2048), (60, 512, 4, 4, 128, 512),
+                                                     (290, 512, 8, 2, 64, 512), (400, 512, 2, 2, 32, 64)])
 def test_attn_decode_rope_oproj_equals_the_two_launches(gpu, pos, max_pos, Hq, Hkv, hd, N):
     """Attention + output projection in one launch (the projection's workgroups fetch their weights while
     the attention runs, then wait for it): attention output, projection output (with the in-place residual)
