@@ -377,6 +377,7 @@ __device__ __forceinline__ void attn_decode_body(const AdArgs &a, float *sc, hal
                                                  int *timeouts = nullptr, const int span_len_arg = 0) {
     static_assert(LS == 256 || LS == 512, "span length");
     const int span_len = span_len_arg > 0 ? span_len_arg : LS; // positions per span (a multiple of 8, at most LS)
+    (void)s_m; // the statistics of a span live in ad_lds_ml; s_l and sc serve the merge of several spans below
     half_t *kst_all = ad_lds_kst<HD>();  // K blocks, one slice per wavefront
     float *ow_all = ad_lds_ow<NDIM, G>();  // unnormalised P.V per wavefront
     float *ml_all = ad_lds_ml<G>();      // (max, sum) per wavefront and head
