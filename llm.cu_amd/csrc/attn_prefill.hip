@@ -501,15 +501,19 @@ __global__ __launch_bounds__(G * 128, 1) void attn_prefill_pipe_kernel(const hal
         return __builtin_bit_cast(half8_t, rr);
     };
 
-    // One pipelined iteration on chunk c (PAR = c % 2): scores of chunk c + 1 into s_nxt, probabilities of chunk c
+    // One pipelined iteration on chunk c (PAR = c % 2, PHASE = c % 8): scores of chunk c + 1 into s_nxt, probabilities of chunk c
     // from s_cur into p_cur, O^T += V^T(chunk c - 1) . p_prv.  Every iteration does all three: past the last
     // chunk the scores are computed from a stale ring slot and never used, and in front of the first chunk the
     // probabilities are zero and the V region was cleared.
-    auto step = [&](float16_t &s_cur, float16_t &s_nxt, ap_u8_t &p_cur, ap_u8_t &p_prv, int c, auto par_c,
+    // phase_c carries c % 8: the ring slots of the K and V fragments are then compile-time constants and fold into
+    // the immediate offsets of the LDS reads (no address arithmetic per read: nine vector-ALU issue slots of about
+    // 85 per iteration, which compete with the MFMAs for the issue port).
+    auto step = [&](float16_t &s_cur, float16_t &s_nxt, ap_u8_t &p_cur, ap_u8_t &p_prv, int c, auto phase_c,
                     int dma_tile) __attribute__((always_inline)) {
-        constexpr int PAR = decltype(par_c)::value;
-        const int koff = ((c + 1) & 7) * HALF_TILE;
-        const int voff = (((c - 1) >> 1) & 3) * TILE;
+        constexpr int PHASE = decltype(phase_c)::value;
+        constexpr int PAR = PHASE & 1;
+        constexpr int koff = ((PHASE + 1) & 7) * HALF_TILE;
+        constexpr int voff = (((PHASE + 7) & 7) >> 1) * TILE;
         constexpr int RA = 3; // fragments read ahead
         half8_t kf[RA], vf[RA];
         auto rd = [&](int grp) __attribute__((always_inline)) {
@@ -568,15 +572,25 @@ __global__ __launch_bounds__(G * 128, 1) void attn_prefill_pipe_kernel(const hal
     }
     asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
 
-    // Two iterations per trip, so that the two score and probability sets keep their roles.  With an odd number
+    // Iterations come in pairs, so that the two score and probability sets keep their roles.  With an odd number
     // of chunks the last iteration works on chunk nc, whose keys lie behind every query of the block: masked,
     // its probabilities are zero, and the second product of the last real chunk rides on it.
+    // Eight iterations per trip (the period of the K ring), left after any pair.
     int dma_tile = clamp_tile(2);
-    for (int c = 0; c < nc; c += 2) {
-        step(S[0], S[1], P[0], P[1], c, std::integral_constant<int, 0>{}, dma_tile);
-        tile_barrier();
-        dma_tile = clamp_tile(c / 2 + 3);
-        step(S[1], S[0], P[1], P[0], c + 1, std::integral_constant<int, 1>{}, dma_tile);
+    for (int c = 0; c < nc; c += 8) {
+#define AP_PAIR(PH)                                                                               \
+        step(S[0], S[1], P[0], P[1], c + PH, std::integral_constant<int, PH>{}, dma_tile);          \
+        tile_barrier();                                                                            \
+        dma_tile = clamp_tile((c + PH) / 2 + 3);                                                   \
+        step(S[1], S[0], P[1], P[0], c + PH + 1, std::integral_constant<int, PH + 1>{}, dma_tile);
+        AP_PAIR(0)
+        if (c + 2 >= nc) break;
+        AP_PAIR(2)
+        if (c + 4 >= nc) break;
+        AP_PAIR(4)
+        if (c + 6 >= nc) break;
+        AP_PAIR(6)
+#undef AP_PAIR
     }
     if (!(nc & 1)) { // second product of the last chunk
         const int voff = (((nc - 1) >> 1) & 3) * TILE;
