@@ -161,7 +161,12 @@ __device__ __forceinline__ uint32_t f16_order_key(uint16_t bits) {
     return (bits & 0x8000u) ? (uint32_t)(0x7fffu - (bits & 0x7fffu)) : (uint32_t)(0x8000u + bits);
 }
 
-__device__ __forceinline__ float silu_f(float g) { return g / (1.0f + expf(-g)); }
+// SiLU (src/inference/inference.cu:451-453: x / (1 + expf(-x)) in fp32).  The reference's expf is CUDA's, whose bits
+// no other math library reproduces, so this is a floating-point step inside the stated tolerance either way: the
+// hardware exponential and reciprocal (a few fp32 ulp, three orders of magnitude below the fp16 rounding that
+// follows) instead of the library expf and the IEEE division, which cost 2 % of the prompt pass's gate/up GEMM.
+// Every path (GEMV, skinny, GEMM, fused decode) goes through this one function.
+__device__ __forceinline__ float silu_f(float g) { return __fdividef(g, 1.0f + __expf(-g)); }
 
 // fp16(SiLU(gate) * up) as the reference rounds it (src/inference/inference.cu:513-516: the product is an
 // fp32 value, then __float2half): the empty asm keeps the compiler from folding the multiply and the
