@@ -202,7 +202,20 @@ __global__ __launch_bounds__(256) void v_append_transpose_kernel(const half_t *_
         for (int j = 0; j < 8; ++j) tile[r][cc + j] = v[j];
     }
     __syncthreads();
-    // write: for column c (a (kvh, dd) pair) positions t0..t0+63 are contiguous in the cache
+    // write: for column c (a (kvh, dd) pair) positions t0..t0+63 are contiguous in the cache.  With whole groups of
+    // eight positions on 16-byte boundaries a thread stores eight of them at once.
+    if (((pos0 + t0) & 7) == 0 && (max_pos & 7) == 0 && ((uintptr_t)vc & 15u) == 0 && t0 + 64 <= T && c0 + 64 <= kvd) {
+        for (int i = threadIdx.x; i < 512; i += 256) {
+            const int cc = i / 8, r8 = (i % 8) * 8;
+            half8_t v;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) v[j] = tile[r8 + j][cc];
+            const int col = c0 + cc;
+            const int kvh = col / head_dim, dd = col % head_dim;
+            store8(vc + ((size_t)kvh * head_dim + dd) * max_pos + pos0 + t0 + r8, v);
+        }
+        return;
+    }
     for (int i = threadIdx.x; i < 64 * 64; i += 256) {
         int cc = i / 64, r = i % 64;
         int col = c0 + cc;
