@@ -24,6 +24,10 @@ HIP_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off",
     # packed-fp32 VALU forms are kept off for every device function
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # the command processor puts a kernel's first 14 argument dwords into scalar registers before its wavefronts
+    # start (scalar and pointer arguments only: the decode kernels take theirs that way), so the first loads do not
+    # wait for a trip to the argument buffer; code objects keep a prologue for firmware without the feature
+    "-mllvm", "-amdgpu-kernarg-preload-count=14",
     "-Wno-unused-command-line-argument", "-Wno-unknown-warning-option",
     "-I", INCLUDE, "-I", os.path.join(HERE, "csrc"),
 ]

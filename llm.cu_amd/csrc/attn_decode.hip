@@ -175,8 +175,27 @@ __device__ __forceinline__ void ao_projection_part(const AdArgs &a, const AoArgs
     }
 }
 
+// Arguments as scalars, what the attention workgroups need for their first loads in front (the first 14 dwords
+// reach the wavefronts in scalar registers, see the build flags; structs passed by value do not).
+// kvh_maxpos = n_kv_heads | max_pos << 8.
 template <int HD, int G, int DSN>
-__global__ __launch_bounds__(AD_THREADS) void attn_oproj_kernel(const AdArgs a, const AoArgs o) {
+__global__ __launch_bounds__(AD_THREADS) void attn_oproj_kernel(const int32_t *pos_dev, const half_t *qkv, half_t *kc,
+                                                                half_t *vc, const float *table, const half_t *w,
+                                                                int pos_host, int kvh_maxpos, half_t *attn_out,
+                                                                const half_t *res, half_t *out, uint16_t *next, int N,
+                                                                int K, int n_owg, int rows, int *timeouts) {
+    AdArgs a = {};
+    a.q = qkv;
+    a.kc = kc;
+    a.vc = vc;
+    a.out = attn_out;
+    a.table = table;
+    a.pos_host = pos_host;
+    a.pos_dev = pos_dev;
+    a.n_kv_heads = kvh_maxpos & 0xff;
+    a.max_pos = (int)((unsigned)kvh_maxpos >> 8);
+    a.splits = 1;
+    const AoArgs o = {w, res, out, next, N, K, n_owg, rows, timeouts};
     __shared__ float sc[G * AD_LS];
     __shared__ __attribute__((aligned(16))) half_t qs[G * HD];
     __shared__ __attribute__((aligned(16))) half_t knew[HD];
@@ -220,7 +239,11 @@ static int launch_attn_oproj(AdArgs a, AoArgs o, hipStream_t s) {
     o.n_owg = owg;
     o.rows = rows;
     a.splits = 1;
-    attn_oproj_kernel<HD, G, DSN><<<dim3(n_attn + owg), dim3(AD_THREADS), 0, s>>>(a, o);
+    LLM_REQUIRE(a.n_kv_heads < 256 && a.max_pos < (1 << 23), "llm_attn_decode_rope_oproj: %d kv heads, max_pos %d", a.n_kv_heads,
+                a.max_pos);
+    attn_oproj_kernel<HD, G, DSN><<<dim3(n_attn + owg), dim3(AD_THREADS), 0, s>>>(
+        a.pos_dev, a.q, a.kc, a.vc, a.table, o.w, a.pos_host, a.n_kv_heads | (a.max_pos << 8), a.out, o.res, o.out, o.next, o.N,
+        o.K, o.n_owg, o.rows, o.timeouts);
     LLM_LAUNCH_CHECK("attn_oproj_kernel");
     return LLM_OK;
 }

@@ -36,8 +36,15 @@ struct GemvArgs {
     int N, K, rpw;
 };
 
+// The arguments travel as scalars, the pointers and sizes that the first loads need in front: the file is built
+// with kernel-argument preloading, which has the command processor put the first 14 dwords into scalar registers
+// before the wavefronts start (a struct passed by value is not preloaded), so the first loads do not wait for a
+// trip to the argument buffer.  n_rpw = N | rows per wavefront << 28.
 template <int MODE>
-__global__ __launch_bounds__(GEMV_THREADS) void gemv_kernel(const GemvArgs a) {
+__global__ __launch_bounds__(GEMV_THREADS) void gemv_kernel(const half_t *x, const half_t *w, const half_t *gain,
+                                                            const half_t *w2, const half_t *res, half_t *out, int n_rpw,
+                                                            int K_arg, double eps, unsigned long long *cand) {
+    const GemvArgs a = {x, gain, eps, w, w2, res, out, cand, n_rpw & 0x0fffffff, K_arg, (int)((unsigned)n_rpw >> 28)};
     constexpr int NW = MODE == GV_SWIGLU ? 2 : 1; // weight streams per row
 #ifndef GEMV_NBUF1
 #define GEMV_NBUF1 2
@@ -263,7 +270,9 @@ template <int MODE> static int gemv_dispatch(GemvArgs a, hipStream_t s) {
     LLM_REQUIRE(a.K % 8 == 0 && smem <= 56 * 1024, "GEMV: K=%d must be a multiple of 8 and fit 56 KiB of LDS", a.K);
     LLM_REQUIRE(!a.gain || (rms_shape_ok(a.K) && a.K <= 4 * GEMV_NORM_R * GEMV_THREADS),
                 "GEMV with RMSNorm: K=%d (need K/4 a power of two in [64, %d])", a.K, GEMV_NORM_R * GEMV_THREADS);
-    gemv_kernel<MODE><<<dim3(gemv_blocks(a.N, a.rpw)), dim3(GEMV_THREADS), smem, s>>>(a);
+    LLM_REQUIRE(a.N < (1 << 28) && a.rpw >= 1 && a.rpw < 16, "GEMV: N=%d rows per wavefront %d", a.N, a.rpw);
+    gemv_kernel<MODE><<<dim3(gemv_blocks(a.N, a.rpw)), dim3(GEMV_THREADS), smem, s>>>(a.x, a.w, a.gain, a.w2, a.res, a.out,
+                                                                                     a.N | (a.rpw << 28), a.K, a.eps, a.cand);
     LLM_LAUNCH_CHECK("gemv_kernel");
     return LLM_OK;
 }
