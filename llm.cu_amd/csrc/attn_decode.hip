@@ -291,8 +291,26 @@ static int dispatch_decode(AdArgs a, int n_heads, int head_dim, void *ws, hipStr
 #define AD_LONG_LS_MAX 512  // longest
 #define AD_MERGE_THREADS 512
 
+// (arguments as leading scalars, like attn_oproj_kernel: kvh_maxpos = n_kv_heads | max_pos << 8,
+// splits_target = splits | span_target << 16)
 template <int HD, int G, bool FUSED>
-__global__ __launch_bounds__(AD_THREADS) void attn_span_kernel(const AdArgs a) {
+__global__ __launch_bounds__(AD_THREADS) void attn_span_kernel(const int32_t *pos_dev, const half_t *q, half_t *kc,
+                                                               half_t *vc, const float *table, int pos_host,
+                                                               int kvh_maxpos, int splits_target, float *ws_acc,
+                                                               float *ws_ml) {
+    AdArgs a = {};
+    a.q = q;
+    a.kc = kc;
+    a.vc = vc;
+    a.table = table;
+    a.pos_host = pos_host;
+    a.pos_dev = pos_dev;
+    a.n_kv_heads = kvh_maxpos & 0xff;
+    a.max_pos = (int)((unsigned)kvh_maxpos >> 8);
+    a.splits = splits_target & 0xffff;
+    a.span_target = (int)((unsigned)splits_target >> 16);
+    a.ws_acc = ws_acc;
+    a.ws_ml = ws_ml;
     __shared__ float sc[G * AD_LONG_LS];
     __shared__ __attribute__((aligned(16))) half_t qs[G * HD];
     __shared__ __attribute__((aligned(16))) half_t knew[HD];
@@ -404,6 +422,8 @@ static int ad_long_setup(AdArgs &a, int *gy) {
     const int splits = (a.max_pos + AD_LONG_LS - 1) / AD_LONG_LS; // spans of the workspace layout: never fewer than in use
     LLM_REQUIRE(splits <= AD_MAX_SPLITS, "decode attention: max_pos=%d exceeds %d", a.max_pos, AD_MAX_SPLITS * AD_LONG_LS);
     a.splits = splits;
+    LLM_REQUIRE(a.n_kv_heads < 256 && a.max_pos < (1 << 23) && a.span_target < (1 << 15), "decode attention: %d kv heads, max_pos %d",
+                a.n_kv_heads, a.max_pos);
     if (a.pos_dev) {
         const int knee = a.span_target * AD_LONG_LS < a.max_pos ? a.span_target * AD_LONG_LS : a.max_pos;
         const int m1 = ad_long_spans(knee, a.span_target), m2 = ad_long_spans(a.max_pos, a.span_target);
@@ -423,7 +443,9 @@ static int launch_decode_long(AdArgs a, void *ws, hipStream_t s) {
     int gy = 0;
     int rc = ad_long_setup(a, &gy);
     if (rc != LLM_OK) return rc;
-    attn_span_kernel<HD, G, FUSED><<<dim3(a.n_kv_heads, gy), dim3(AD_THREADS), 0, s>>>(a);
+    attn_span_kernel<HD, G, FUSED><<<dim3(a.n_kv_heads, gy), dim3(AD_THREADS), 0, s>>>(
+        a.pos_dev, a.q, a.kc, a.vc, a.table, a.pos_host, a.n_kv_heads | (a.max_pos << 8), a.splits | (a.span_target << 16), a.ws_acc,
+        a.ws_ml);
     LLM_LAUNCH_CHECK("attn_span_kernel");
     attn_merge_kernel<HD, G><<<dim3(Hq), dim3(AD_MERGE_THREADS), 0, s>>>(a);
     LLM_LAUNCH_CHECK("attn_merge_kernel");
@@ -438,7 +460,22 @@ static int launch_decode_long(AdArgs a, void *ws, hipStream_t s) {
 // and the projection needs no launch of its own.
 // ---------------------------------------------------------------------------
 template <int HD, int G>
-__global__ __launch_bounds__(AD_THREADS) void merge_oproj_kernel(const AdArgs a, const AoArgs o) {
+__global__ __launch_bounds__(AD_THREADS) void merge_oproj_kernel(const int32_t *pos_dev, const float *ws_ml,
+                                                                 const float *ws_acc, const half_t *w, int pos_host,
+                                                                 int kvh_maxpos, int splits_target, int N, int K, int n_owg,
+                                                                 half_t *attn_out, const half_t *res, half_t *out,
+                                                                 uint16_t *next, int rows, int *timeouts) {
+    AdArgs a = {};
+    a.out = attn_out;
+    a.pos_host = pos_host;
+    a.pos_dev = pos_dev;
+    a.n_kv_heads = kvh_maxpos & 0xff;
+    a.max_pos = (int)((unsigned)kvh_maxpos >> 8);
+    a.splits = splits_target & 0xffff;
+    a.span_target = (int)((unsigned)splits_target >> 16);
+    a.ws_acc = const_cast<float *>(ws_acc);
+    a.ws_ml = const_cast<float *>(ws_ml);
+    const AoArgs o = {w, res, out, next, N, K, n_owg, rows, timeouts};
     static_assert(AD_MERGE_THREADS == AD_THREADS, "both roles share the workgroup size");
     __shared__ __attribute__((aligned(16))) half_t xs[AO_KSTEPS * 512];
     const int n_first = a.n_kv_heads * G;
@@ -477,9 +514,13 @@ static int launch_long_oproj(AdArgs a, AoArgs o, void *ws, hipStream_t s) {
     int gy = 0;
     rc = ad_long_setup(a, &gy);
     if (rc != LLM_OK) return rc;
-    attn_span_kernel<HD, G, true><<<dim3(a.n_kv_heads, gy), dim3(AD_THREADS), 0, s>>>(a);
+    attn_span_kernel<HD, G, true><<<dim3(a.n_kv_heads, gy), dim3(AD_THREADS), 0, s>>>(
+        a.pos_dev, a.q, a.kc, a.vc, a.table, a.pos_host, a.n_kv_heads | (a.max_pos << 8), a.splits | (a.span_target << 16), a.ws_acc,
+        a.ws_ml);
     LLM_LAUNCH_CHECK("attn_span_kernel");
-    merge_oproj_kernel<HD, G><<<dim3(Hq + o.n_owg), dim3(AD_THREADS), 0, s>>>(a, o);
+    merge_oproj_kernel<HD, G><<<dim3(Hq + o.n_owg), dim3(AD_THREADS), 0, s>>>(
+        a.pos_dev, a.ws_ml, a.ws_acc, o.w, a.pos_host, a.n_kv_heads | (a.max_pos << 8), a.splits | (a.span_target << 16), o.N, o.K,
+        o.n_owg, a.out, o.res, o.out, o.next, o.rows, o.timeouts);
     LLM_LAUNCH_CHECK("merge_oproj_kernel");
     return LLM_OK;
 }
