@@ -101,9 +101,10 @@ __device__ __forceinline__ void ao_projection_part(const AdArgs &a, const AoArgs
     const int wtotal = o.n_owg * AO_WAVES;
     half8_t wreg[AO_ROWS][AO_KSTEPS];
     half_t resv[AO_ROWS];
-    // a head start of about a microsecond for the attention's own loads (measured: 12.2 -> 11.4 us per launch)
+    // a head start of a little under a microsecond for the attention's own loads (measured per launch: 12.2 -> 11.4 us
+    // with the first version of the attention; against the current one three pauses beat 0-2 and 4-8)
 #ifndef AO_HEAD_START
-#define AO_HEAD_START 5
+#define AO_HEAD_START 3
 #endif
     for (int dl = 0; dl < AO_HEAD_START; ++dl) __builtin_amdgcn_s_sleep(8);
 #pragma unroll
