@@ -97,7 +97,11 @@ __device__ __forceinline__ void ao_projection_part(const AdArgs &a, const AoArgs
     const int wg = blockIdx.x, tid = threadIdx.x;
     const int wave = tid / 64, lane = tid % 64;
     const int K = o.K, N = o.N;
-    const int wslot = (wg - n_attn) * AO_WAVES + wave; // this wavefront among all of the projection part
+    // Row i of projection workgroup p is p + n_owg * i (adjacent workgroups read adjacent rows at the same time), dealt
+    // to its wavefronts in turn: every workgroup, i.e. every CU, streams N / n_owg rows to within one (18 or 19 of the
+    // 8B model's 4096 on 224 CUs), where rows dealt wavefront by wavefront over the whole launch left 24 to some CUs
+    // and 16 to the others.
+    const int wslot = (wg - n_attn) + o.n_owg * wave;
     const int wtotal = o.n_owg * AO_WAVES;
     half8_t wreg[AO_ROWS][AO_KSTEPS];
     half_t resv[AO_ROWS];
@@ -109,7 +113,7 @@ __device__ __forceinline__ void ao_projection_part(const AdArgs &a, const AoArgs
     for (int dl = 0; dl < AO_HEAD_START; ++dl) __builtin_amdgcn_s_sleep(8);
 #pragma unroll
     for (int r = 0; r < AO_ROWS; ++r) {
-        int row = wslot + wtotal * r; // adjacent wavefronts read adjacent rows
+        int row = wslot + wtotal * r;
         const bool live = r < o.rows && row < N;
         row = live ? row : N - 1;
 #pragma unroll
