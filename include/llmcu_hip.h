@@ -141,6 +141,16 @@ int llm_norm_linear_swiglu(const uint16_t *x_dev, const uint16_t *gain_dev, doub
                            const uint16_t *wgate_dev, const uint16_t *wup_dev, uint16_t *out_dev, int N,
                            int K, llm_stream_t stream);
 
+/* The first projection of a decode step with the embedding gather folded in: the input row is
+ * table[ids[ids_offset ? *ids_offset : 0]] (a row of 0x7fff NaNs for an id outside [0, vocab), as
+ * llm_embed_gather writes), out = linear(rmsnorm(row, gain, eps), w), and x_out receives the row itself (the
+ * residual stream of the first layer).  Replaces tokens_to_embeddings followed by compute_layer_norm and
+ * compute_qkv_tensors of layer 0 (src/inference/inference.cu:149-163) for T = 1; same bits as
+ * llm_embed_gather followed by llm_norm_linear, one launch fewer. */
+int llm_embed_norm_linear(const uint16_t *table_dev, const int32_t *ids_dev, const int32_t *ids_offset_dev, int vocab,
+                          uint16_t *x_out_dev, const uint16_t *gain_dev, double eps, const uint16_t *w_dev,
+                          uint16_t *out_dev, int N, int K, llm_stream_t stream);
+
 /* ---- attention ------------------------------------------------------------------ */
 /* Replaces compute_attention and its three kernels
  * (src/inference/inference.cu:698-947) for one new row: causal GQA attention

@@ -127,6 +127,7 @@ HIP_ABI = {
     "llm_linear_swiglu": (_i, [_vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
     "llm_norm_linear": (_i, [_vp, _vp, C.c_double, _vp, _vp, _i, _i, _vp]),
     "llm_norm_linear_swiglu": (_i, [_vp, _vp, C.c_double, _vp, _vp, _vp, _i, _i, _vp]),
+    "llm_embed_norm_linear": (_i, [_vp, _vp, _vp, _i, _vp, _vp, C.c_double, _vp, _vp, _i, _i, _vp]),
     "llm_attn_decode_rope": (_i, [_vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _vp, _vp]),
     "llm_attn_decode_rope_batch": (_i, [_vp, _i, _vp, _vp, _vp, _i, _vp, _i, _vp, _i, _i, _i, _i, _vp, _vp]),
     "llm_attn_oproj_supported": (_i, [_i, _i, _i, _i]),

@@ -24,6 +24,8 @@ int gemv_launch(const half_t *x, const half_t *gain, double eps, const half_t *w
                 int N, int K, hipStream_t s);
 int gemv_swiglu_launch(const half_t *x, const half_t *gain, double eps, const half_t *wg, const half_t *wu,
                        half_t *out, int N, int K, hipStream_t s);
+int gemv_embed_launch(const half_t *table, const int32_t *ids, const int32_t *ids_offset, int vocab, half_t *x_copy,
+                      const half_t *gain, double eps, const half_t *w, half_t *out, int N, int K, hipStream_t s);
 
 
 // address-space cast for the LDS side of the loads that go from global memory straight into LDS
@@ -1185,6 +1187,17 @@ int llm_norm_linear(const uint16_t *x, const uint16_t *gain, double eps, const u
     LLM_REQUIRE(aligned16(x) && aligned16(gain) && aligned16(w), "llm_norm_linear: pointers must be 16-byte aligned");
     return gemv_launch((const half_t *)x, (const half_t *)gain, eps, (const half_t *)w, nullptr, (half_t *)out, N, K,
                        (hipStream_t)stream);
+}
+
+int llm_embed_norm_linear(const uint16_t *table, const int32_t *ids, const int32_t *ids_offset, int vocab, uint16_t *x_out,
+                          const uint16_t *gain, double eps, const uint16_t *w, uint16_t *out, int N, int K,
+                          llm_stream_t stream) {
+    LLM_REQUIRE(table && ids && x_out && gain && w && out, "llm_embed_norm_linear: null pointer");
+    LLM_REQUIRE(N > 0 && K > 0 && vocab > 0, "llm_embed_norm_linear: N=%d K=%d vocab=%d", N, K, vocab);
+    LLM_REQUIRE(aligned16(table) && aligned16(gain) && aligned16(w) && aligned16(x_out),
+                "llm_embed_norm_linear: pointers must be 16-byte aligned");
+    return gemv_embed_launch((const half_t *)table, ids, ids_offset, vocab, (half_t *)x_out, (const half_t *)gain, eps,
+                             (const half_t *)w, (half_t *)out, N, K, (hipStream_t)stream);
 }
 
 int llm_norm_linear_swiglu(const uint16_t *x, const uint16_t *gain, double eps, const uint16_t *wgate,

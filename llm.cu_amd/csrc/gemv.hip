@@ -22,7 +22,9 @@
 #define GEMV_SPAN (512 * GEMV_U)
 #define GEMV_NORM_R 4 // fused RMSNorm: K <= 4 * 4 * GEMV_THREADS = 4096
 
-enum { GV_PLAIN = 0, GV_SWIGLU = 1, GV_LMHEAD = 2 };
+// GV_EMBED: GV_PLAIN whose input vector is a row of an embedding table, picked by a token id in device memory
+// (the first projection of a decode step: the gather costs no launch of its own).
+enum { GV_PLAIN = 0, GV_SWIGLU = 1, GV_LMHEAD = 2, GV_EMBED = 3 };
 
 struct GemvArgs {
     const half_t *x;     // [K]
@@ -34,6 +36,11 @@ struct GemvArgs {
     half_t *out;         // [N] (GV_LMHEAD: the fp16 logits)
     unsigned long long *cand; // GV_LMHEAD: one argmax candidate per workgroup
     int N, K, rpw;
+    // GV_EMBED: x is the table [vocab, K]; the row is ids[ids_offset ? *ids_offset : 0] (a NaN row for an id outside
+    // [0, vocab)), and workgroup 0 leaves a copy of it in x_copy (the residual stream of the layer)
+    const int32_t *ids, *ids_offset;
+    half_t *x_copy;
+    int vocab;
 };
 
 // The arguments travel as scalars, the pointers and sizes that the first loads need in front: the file is built
@@ -43,9 +50,13 @@ struct GemvArgs {
 template <int MODE>
 __global__ __launch_bounds__(GEMV_THREADS) void gemv_kernel(const half_t *x, const half_t *w, const half_t *gain,
                                                             const half_t *w2, const half_t *res, half_t *out, int n_rpw,
-                                                            int K_arg, double eps, unsigned long long *cand) {
-    const GemvArgs a = {x, gain, eps, w, w2, res, out, cand, n_rpw & 0x0fffffff, K_arg, (int)((unsigned)n_rpw >> 28)};
+                                                            int K_arg, double eps, unsigned long long *cand,
+                                                            const int32_t *ids, const int32_t *ids_offset,
+                                                            half_t *x_copy, int vocab) {
+    const GemvArgs a = {x,     gain, eps, w, w2, res, out, cand, n_rpw & 0x0fffffff, K_arg, (int)((unsigned)n_rpw >> 28),
+                        ids,   ids_offset, x_copy, vocab};
     constexpr int NW = MODE == GV_SWIGLU ? 2 : 1; // weight streams per row
+    constexpr bool PLAIN = MODE == GV_PLAIN || MODE == GV_EMBED;
 #ifndef GEMV_NBUF1
 #define GEMV_NBUF1 2
 #endif
@@ -94,7 +105,20 @@ __global__ __launch_bounds__(GEMV_THREADS) void gemv_kernel(const half_t *x, con
 #define GEMV_XRAW 8
 #endif
     half8_t xraw[GEMV_XRAW]; // the first GEMV_XRAW * 2048 elements of a plain input vector, asked for before the weights
-    if (a.gain) {
+    if (MODE == GV_EMBED) {
+        // the weights do not depend on the token: they go out first, the two dependent loads of the id (position,
+        // then id) and the table row follow behind them
+#pragma unroll
+        for (int b = 0; b < NBUF; ++b) issue_next(b);
+        const int id = a.ids[a.ids_offset ? a.ids_offset[0] : 0];
+        const bool ok = id >= 0 && id < a.vocab;
+        rms_load<GEMV_THREADS, GEMV_NORM_R>(a.x + (size_t)(ok ? id : 0) * K, a.gain, K, xr);
+        if (!ok) {
+            const half_t nanv = __builtin_bit_cast(half_t, (uint16_t)0x7fffu);
+#pragma unroll
+            for (int j = 0; j < GEMV_NORM_R; ++j) xr.x[j] = half4_t{nanv, nanv, nanv, nanv};
+        }
+    } else if (a.gain) {
         rms_load<GEMV_THREADS, GEMV_NORM_R>(a.x, a.gain, K, xr);
     } else {
 #pragma unroll
@@ -103,14 +127,16 @@ __global__ __launch_bounds__(GEMV_THREADS) void gemv_kernel(const half_t *x, con
             if (c < K) xraw[j] = load8(a.x + c);
         }
     }
+    if (MODE != GV_EMBED) {
 #pragma unroll
-    for (int b = 0; b < NBUF; ++b) issue_next(b);
+        for (int b = 0; b < NBUF; ++b) issue_next(b);
+    }
     // the residual of each of this wavefront's rows, asked for now: at the end of a row the value is
     // there instead of one more trip to memory behind the last weight load
     // (four named registers and a select chain below: an array indexed by the row counter would live in
     // scratch memory)
     half_t res0 = (half_t)0.f, res1 = (half_t)0.f, res2 = (half_t)0.f, res3 = (half_t)0.f;
-    if (MODE == GV_PLAIN && a.res) {
+    if (PLAIN && a.res) {
         auto ask = [&](int r) {
             const int row = row_base + row_step * r;
             return (r < a.rpw && row < N) ? a.res[row] : (half_t)0.f;
@@ -120,8 +146,13 @@ __global__ __launch_bounds__(GEMV_THREADS) void gemv_kernel(const half_t *x, con
         res2 = ask(2);
         res3 = ask(3);
     }
-    if (a.gain) {
+    if (MODE == GV_EMBED || a.gain) {
         rms_finish<GEMV_THREADS, GEMV_NORM_R>(xr, xs, K, a.eps, red);
+        if (MODE == GV_EMBED && blockIdx.x == 0) {
+#pragma unroll
+            for (int j = 0; j < GEMV_NORM_R; ++j)
+                if (j < xr.R) *reinterpret_cast<half4_t *>(a.x_copy + 4 * (size_t)(threadIdx.x + GEMV_THREADS * j)) = xr.x[j];
+        }
     } else {
 #pragma unroll
         for (int j = 0; j < GEMV_XRAW; ++j) {
@@ -259,7 +290,7 @@ static int rows_per_wave(int mode, int N, bool norm) {
 #define GEMV_RPW_QKV 2
 #endif
     if (mode == GV_LMHEAD) return N >= 32768 ? GEMV_RPW_LM : 1;
-    if (mode == GV_PLAIN && norm && N >= 6144) return GEMV_RPW_QKV;
+    if ((mode == GV_PLAIN || mode == GV_EMBED) && norm && N >= 6144) return GEMV_RPW_QKV;
     return 1;
 }
 
@@ -268,11 +299,13 @@ static int gemv_blocks(int N, int rpw) { return (N + GEMV_WAVES * rpw - 1) / (GE
 template <int MODE> static int gemv_dispatch(GemvArgs a, hipStream_t s) {
     const size_t smem = (size_t)a.K * sizeof(half_t);
     LLM_REQUIRE(a.K % 8 == 0 && smem <= 56 * 1024, "GEMV: K=%d must be a multiple of 8 and fit 56 KiB of LDS", a.K);
+    LLM_REQUIRE(MODE != GV_EMBED || (a.gain && a.ids && a.x_copy && a.vocab > 0), "GEMV on an embedding row: gain, ids, copy, vocab");
     LLM_REQUIRE(!a.gain || (rms_shape_ok(a.K) && a.K <= 4 * GEMV_NORM_R * GEMV_THREADS),
                 "GEMV with RMSNorm: K=%d (need K/4 a power of two in [64, %d])", a.K, GEMV_NORM_R * GEMV_THREADS);
     LLM_REQUIRE(a.N < (1 << 28) && a.rpw >= 1 && a.rpw < 16, "GEMV: N=%d rows per wavefront %d", a.N, a.rpw);
     gemv_kernel<MODE><<<dim3(gemv_blocks(a.N, a.rpw)), dim3(GEMV_THREADS), smem, s>>>(a.x, a.w, a.gain, a.w2, a.res, a.out,
-                                                                                     a.N | (a.rpw << 28), a.K, a.eps, a.cand);
+                                                                                     a.N | (a.rpw << 28), a.K, a.eps, a.cand,
+                                                                                     a.ids, a.ids_offset, a.x_copy, a.vocab);
     LLM_LAUNCH_CHECK("gemv_kernel");
     return LLM_OK;
 }
@@ -281,6 +314,13 @@ int gemv_launch(const half_t *x, const half_t *gain, double eps, const half_t *w
                 int N, int K, hipStream_t s) {
     GemvArgs a = {x, gain, eps, w, nullptr, res, out, nullptr, N, K, rows_per_wave(GV_PLAIN, N, gain != nullptr)};
     return gemv_dispatch<GV_PLAIN>(a, s);
+}
+
+int gemv_embed_launch(const half_t *table, const int32_t *ids, const int32_t *ids_offset, int vocab, half_t *x_copy,
+                      const half_t *gain, double eps, const half_t *w, half_t *out, int N, int K, hipStream_t s) {
+    GemvArgs a = {table, gain, eps, w, nullptr, nullptr, out, nullptr, N, K, rows_per_wave(GV_EMBED, N, true),
+                  ids,   ids_offset, x_copy, vocab};
+    return gemv_dispatch<GV_EMBED>(a, s);
 }
 
 int gemv_swiglu_launch(const half_t *x, const half_t *gain, double eps, const half_t *wg, const half_t *wu,

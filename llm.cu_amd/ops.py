@@ -230,6 +230,20 @@ def norm_linear(x, gain, w, eps=1e-5):
     return d_o.download()
 
 
+def embed_norm_linear(table, ids, offset, gain, w, eps=1e-5):
+    """Returns (out [1, N], the gathered row [K]) for the id at ids[offset] (offset None: ids[0])."""
+    table, gain, w = _u16(table), _u16(gain), _u16(w)
+    vocab, K = table.shape
+    N = w.shape[0]
+    d_t, d_g, d_w = DevBuf.from_host(table), DevBuf.from_host(gain), DevBuf.from_host(w)
+    d_ids = DevBuf.from_host(np.ascontiguousarray(ids, dtype=np.int32))
+    d_off = DevBuf.from_host(np.array([offset], dtype=np.int32)) if offset is not None else None
+    d_x, d_o = DevBuf((K,), np.uint16), DevBuf((1, N), np.uint16)
+    check(lib().llm_embed_norm_linear(d_t.ptr, d_ids.ptr, d_off.ptr if d_off else None, vocab, d_x.ptr, d_g.ptr, eps,
+                                      d_w.ptr, d_o.ptr, N, K, None))
+    return d_o.download(), d_x.download()
+
+
 def norm_linear_swiglu(x, gain, wgate, wup, eps=1e-5):
     x, gain, wgate, wup = _u16(x).reshape(-1), _u16(gain), _u16(wgate), _u16(wup)
     N, K = wgate.shape

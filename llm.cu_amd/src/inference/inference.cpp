@@ -199,8 +199,15 @@ void issue_pass(Engine *e, const Llama3 *m, int T, int pos0, bool dev_pos, bool 
     const int32_t *pd = dev_pos ? e->d_pos : nullptr;
     const int p0 = dev_pos ? 0 : pos0;
 
-    llama3_check(llm_embed_gather(m->embed_tokens->d_fp16_tensor, e->d_tokens + p0, pd, e->x, T, d, c.vocab, s),
-                 "llm_embed_gather");
+    // decode step over a fused Q/K/V matrix: the first projection gathers the embedding row itself
+    bool embed_folded = false;
+    if (T == 1 && c.n_layers > 0) {
+        const LayerW w0 = layer_w(m, 0);
+        embed_folded = w0.wk == w0.wq + (size_t)qd * d && w0.wv == w0.wk + (size_t)kvd * d;
+    }
+    if (!embed_folded)
+        llama3_check(llm_embed_gather(m->embed_tokens->d_fp16_tensor, e->d_tokens + p0, pd, e->x, T, d, c.vocab, s),
+                     "llm_embed_gather");
     const llm_half *final_gain = m->norm->d_fp16_tensor;
     if (T == 1) {
         // decode step: 4 launches per layer, 5 at long contexts (norm folded into the projections, RoPE + cache
@@ -211,7 +218,11 @@ void issue_pass(Engine *e, const Llama3 *m, int T, int pos0, bool dev_pos, bool 
             if (inject && l > 0)
                 llama3_check(llm_memcpy_d2d(e->x, e->inject_dev + (size_t)(l - 1) * d, sizeof(llm_half) * (size_t)d, s),
                              "inject copy");
-            if (w.wk == w.wq + (size_t)qd * d && w.wv == w.wk + (size_t)kvd * d) {
+            if (l == 0 && embed_folded) {
+                llama3_check(llm_embed_norm_linear(m->embed_tokens->d_fp16_tensor, e->d_tokens + p0, pd, c.vocab, e->x,
+                                                   w.in_ln, c.rms_eps, w.wq, e->qkv, QKV, d, s),
+                             "llm_embed_norm_linear(qkv)");
+            } else if (w.wk == w.wq + (size_t)qd * d && w.wv == w.wk + (size_t)kvd * d) {
                 llama3_check(llm_norm_linear(e->x, w.in_ln, c.rms_eps, w.wq, e->qkv, QKV, d, s), "llm_norm_linear(qkv)");
             } else {
                 llama3_check(llm_norm_linear(e->x, w.in_ln, c.rms_eps, w.wq, e->qkv, qd, d, s), "llm_norm_linear(q)");

@@ -492,6 +492,32 @@ def test_norm_linear_equals_rmsnorm_then_linear(gpu, K, N):
     assert H.mixed_err(got, orc.linear(orc.rmsnorm(x, g), w)) <= TIGHT
 
 
+@pytest.mark.parametrize("K,N,vocab", [(4096, 6144, 1000), (256, 384, 50), (4096, 100, 7)])
+def test_embed_norm_linear_equals_gather_then_norm_linear(gpu, K, N, vocab):
+    """The first projection of a decode step with the gather folded in: the row it leaves is the table's row, the
+    projection has the bits of llm_embed_gather + llm_norm_linear, the id is read at ids[*offset], and an id
+    outside the table gives the gather's NaN row and a NaN projection."""
+    rng = np.random.default_rng(K + N)
+    table = H.bits(2.0 * rng.standard_normal((vocab, K)))
+    g = H.bits(1.0 + 0.1 * rng.standard_normal(K))
+    w = H.bits(0.02 * rng.standard_normal((N, K), dtype=np.float32))
+    ids = np.array([3, vocab - 1, 0, vocab, -1, 5], np.int32)
+    for off in (None, 0, 1, 2, 5):
+        say("embed_norm_linear", K, N, vocab, "offset", off)
+        tok = int(ids[off or 0])
+        got, row = gpu.ops.embed_norm_linear(table, ids, off, g, w)
+        assert np.array_equal(row, table[tok])
+        x = gpu.ops.embed_gather(table, np.array([tok], np.int32))
+        assert np.array_equal(got, gpu.ops.norm_linear(x, g, w))
+        assert H.mixed_err(got, orc.linear(orc.rmsnorm(orc.embed(table, [tok]), g), w)) <= TIGHT
+    for off in (3, 4):
+        say("embed_norm_linear", K, N, vocab, "bad id at offset", off)
+        got, row = gpu.ops.embed_norm_linear(table, ids, off, g, w)
+        assert np.all(row == 0x7fff)
+        x = gpu.ops.embed_gather(table, ids[off:off + 1])
+        assert np.array_equal(got, gpu.ops.norm_linear(x, g, w)) and np.all(np.isnan(H.f16(got)))
+
+
 @pytest.mark.parametrize("K,N", [(4096, 14336), (256, 768)])
 def test_norm_linear_swiglu_equals_unfused(gpu, K, N):
     rng = np.random.default_rng(K + 1)
