@@ -900,10 +900,27 @@ __global__ __launch_bounds__(256, 1) void gemm_dma64_kernel(const half_t *__rest
                       (!(NB == 1 && res) || (((uintptr_t)res & 15u) == 0 && ldr % 8 == 0));
     if (wide) {
         const int g = lane / 16;
+        // The residual values of the whole tile are asked for before the first store: out may be res itself (the
+        // engine adds in place), so a load inside the store loop would have to wait behind the store before it,
+        // one trip to memory per 16 bytes.  A thread reads exactly the elements it writes, so reading them all
+        // first is the same computation.
+        half8_t rv_all[NB == 1 ? 8 : 1][NB == 1 ? 4 : 1];
+        if (NB == 1 && res) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const int m = m0 + wm * WTM + i * 16 + mrow;
+                const int mc = m < T ? m : T - 1;
+#pragma unroll
+                for (int jp = 0; jp < 4; ++jp) {
+                    const int n = n0 + wn * 128 + 16 * (2 * jp + (g & 1)) + 8 * (g >> 1);
+                    const int nc = n < N ? n : N - 8;
+                    rv_all[NB == 1 ? i : 0][NB == 1 ? jp : 0] = load8(res + (size_t)mc * ldr + nc);
+                }
+            }
+        }
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
             const int m = m0 + wm * WTM + i * 16 + mrow;
-            const int mc = m < T ? m : T - 1;
 #pragma unroll
             for (int jp = 0; jp < 4 / NB; ++jp) {
                 const uint2_t a = __builtin_bit_cast(uint2_t, product(2 * jp, i));
@@ -915,8 +932,7 @@ __global__ __launch_bounds__(256, 1) void gemm_dma64_kernel(const half_t *__rest
                 half8_t h = __builtin_bit_cast(half8_t, packed);
                 const int n = n0 + (NB == 1 ? wn * 128 : wn * 64) + 16 * (2 * jp + (g & 1)) + 8 * (g >> 1);
                 if (NB == 1 && res) {
-                    const int nc = n < N ? n : N - 8;
-                    const half8_t rv = load8(res + (size_t)mc * ldr + nc);
+                    const half8_t rv = rv_all[NB == 1 ? i : 0][NB == 1 ? jp : 0];
 #pragma unroll
                     for (int e = 0; e < 8; ++e) h[e] = (half_t)((float)h[e] + (float)rv[e]);
                 }
