@@ -286,6 +286,12 @@ def power_ceiling(pkg, a):
     random operands, then the 8192-token prompt pass and its gate/up GEMM, each for a second or more with amd-smi
     sampled alongside.  Prints one JSON object."""
     lib, eng_mod = pkg.lib(), pkg.engine
+    probe_path = os.path.join(os.path.dirname(pkg.capi.LIB_PATH), "libllmcu_probe.so")
+    if not os.path.exists(probe_path):
+        raise RuntimeError("%s is missing: run `python llm.cu_amd/build.py`" % probe_path)
+    probe = C.CDLL(probe_path)
+    probe.mfma_probe.restype = C.c_int
+    probe.mfma_probe.argtypes = [C.c_int, C.c_float, C.POINTER(C.c_double), C.POINTER(C.c_float)]
     res = {}
     with SmiSampler() as smi:
         time.sleep(1.0)
@@ -294,7 +300,9 @@ def power_ceiling(pkg, a):
                            (2, "mfma_16x16x32_only_constant_operands"), (3, "mfma_16x16x32_only_random_operands")):
             tf, ms = C.c_double(0), C.c_float(0)
             t0 = time.time()
-            pkg.capi.check(lib.llm_mfma_probe(kind, C.c_float(2500.0), C.byref(tf), C.byref(ms), None))
+            rc = probe.mfma_probe(kind, C.c_float(2500.0), C.byref(tf), C.byref(ms))
+            if rc != 0:
+                raise RuntimeError("mfma_probe(kind %d) failed with code %d" % (kind, rc))
             res[name] = dict(tflops=tf.value, frac_of_2500=tf.value / 2500.0, ms=ms.value, **smi.window(t0, time.time()))
             log(name, res[name])
             time.sleep(1.0)

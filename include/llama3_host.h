@@ -167,15 +167,6 @@ void llama3_set_device_sampling(CudaCache *c, int on);
 void llama3_sampler_draw_counts(const CudaCache *c, long *device_draws, long *host_draws);
 /* The cache's sampler (settings, device selection) applied to fp16 logits [vocab] in device memory. */
 int llama3_sample_device_logits(CudaCache *c, const llm_half *logits_dev);
-/* 1: decode steps below 512 cached positions run as one launch per token (llm_decode_fused) when the
- * model shapes and the device allow it; 0 (default): one launch per operation.  Same results bit for
- * bit; on MI355X the per-operation launches are the faster of the two (305 against 361 tok/s at 8B). */
-void llama3_set_fused_decode(CudaCache *c, int on);
-int llama3_fused_decode_active(const CudaCache *c);
-/* The vectors the last one-launch token passed between its phases, all layers: which = 0 qkv, 1 attention
- * output, 2 x after O, 3 FFN hidden vector, 4 layer output; out: [n_layers][width] fp16. */
-void llama3_read_fused_vectors(CudaCache *c, int which, llm_half *out);
-
 typedef struct {
     int n_layers;
     int d_model;
@@ -247,6 +238,21 @@ void llama3_set_hidden_inject(CudaCache *c, const llm_half *hidden);
 /* Choose between one hipGraph replay per decode step (1, default) and plain
  * stream launches (0). */
 void llama3_set_use_graph(CudaCache *c, int on);
+
+/* The decode step's launches that hand the attention output to the output projection inside one kernel
+ * (llm_attn_decode_rope_oproj, llm_attn_decode_rope_long_oproj) bound the projection's wait.  When a wait
+ * gives up -- only seen when other work holds the device's CUs for the whole wait -- the step's results are
+ * discarded, the step (for llama3_generate: its run of decode steps) is redone with one launch per
+ * operation, a line goes to stderr, and the cache keeps the one-launch-per-operation form from then on:
+ * the same token ids either way, a slower step instead of a failed one.
+ * llama3_set_handover: on = 1 puts a cache back into the hand-over form (0 takes it out); spin_limit is
+ * the bound of the wait in polling rounds, negative for the kernels' default.
+ * llama3_handover_stats: waits that gave up and steps redone so far, and whether the form is in use.
+ * llama3_test_mark_handover_timeout: the next step is treated as if one wait had given up (for tests of
+ * the redo path; every kernel still runs to its normal end). */
+void llama3_set_handover(CudaCache *c, int on, int spin_limit);
+void llama3_handover_stats(const CudaCache *c, long *timeouts, long *recoveries, int *active);
+void llama3_test_mark_handover_timeout(CudaCache *c);
 
 /* Error hook.  Default prints the message and calls exit(1) as the reference
  * does; tests install a handler that records instead. */

@@ -40,6 +40,7 @@ int llm_device_name(char *buf, size_t n); /* e.g. "gfx950:sramecc+:xnack-" */
 int llm_device_cu_count(int *n);
 int llm_malloc(void **ptr, size_t bytes);           /* cudaMalloc   (inference.cu:101-108) */
 int llm_free(void *ptr);                            /* cudaFree */
+int llm_mem_info(size_t *free_bytes, size_t *total_bytes); /* cudaMemGetInfo (inference.cu:46-62) */
 int llm_malloc_host(void **ptr, size_t bytes);      /* pinned host memory */
 int llm_free_host(void *ptr);
 int llm_memcpy_h2d(void *dst, const void *src, size_t bytes, llm_stream_t stream);
@@ -197,7 +198,15 @@ int llm_attn_decode_rope(const uint16_t *qkv_dev, uint16_t *k_cache_dev, uint16_
  * attn_out_dev must hold the "empty" pattern when the launch starts: llm_attn_oproj_buffer_init() once,
  * after that every launch refills attn_out_next_dev, the buffer that the next such launch in stream
  * order will pass as attn_out_dev (a ring of two or more buffers; never the same as attn_out_dev).
- * timeouts_dev: one int32, zeroed by the caller, counts waits that gave up (must stay 0).
+ * The wait of the projection workgroups is bounded: after spin_limit polling rounds (a negative value selects
+ * the default, 2^18 rounds, a few tenths of a second) a workgroup gives up, reduces whatever the buffer holds
+ * and adds one to *timeouts_dev (one int32, zeroed by the caller).  A non-zero count after the launch means
+ * out_dev is invalid: fill attn_out_dev and attn_out_next_dev with llm_attn_oproj_buffer_init again, zero the
+ * count and redo the operation (llm_attn_decode_rope + llm_linear give the same bits).  The wait relies on the
+ * hardware handing out the workgroups of a launch in id order, so the attention workgroups run before any
+ * projection workgroup waits for them; that also holds when launches of several streams share the device.
+ * Something else that keeps every CU busy for the whole wait (another process's long kernel) shows up as a
+ * counted timeout, never as a hang.
  * Launches that share these buffers must not overlap.  Limits: Hq*hd <= 4096, N <= 24 * (CUs - Hkv*4). */
 int llm_attn_oproj_supported(int n_heads, int n_kv_heads, int head_dim, int N); /* 1 or 0, current device */
 int llm_attn_oproj_buffer_init(uint16_t *buf_dev, int n, llm_stream_t stream);
@@ -205,7 +214,7 @@ int llm_attn_decode_rope_oproj(const uint16_t *qkv_dev, uint16_t *k_cache_dev, u
                                uint16_t *attn_out_dev, uint16_t *attn_out_next_dev, int pos_host,
                                const int32_t *pos_dev, const float *table_dev, int n_heads, int n_kv_heads,
                                int head_dim, int max_pos, const uint16_t *w_dev, const uint16_t *residual_dev,
-                               uint16_t *out_dev, int N, int32_t *timeouts_dev, llm_stream_t stream);
+                               uint16_t *out_dev, int N, int32_t *timeouts_dev, int spin_limit, llm_stream_t stream);
 /* The same operation as two launches: one workgroup per (KV head, 256-position span) leaves partial
  * softmax statistics and P.V, a second kernel (one workgroup per query head) merges them.  Correct at
  * any position; faster than the single launch beyond 512 cached positions (no in-kernel merge tail). */
@@ -216,7 +225,7 @@ int llm_attn_decode_rope_long(const uint16_t *qkv_dev, uint16_t *k_cache_dev, ui
 /* llm_attn_decode_rope_long and the projection that consumes its result in two launches instead of three
  * (compute_output + add_norm, src/inference/inference.cu:600-618,366-390): the span kernel as above, then one
  * launch whose first Hq workgroups merge one query head each while all others fetch their rows of w and wait
- * for the merged vector.  Buffers, hand-over, timeouts_dev and the bits of the result as for
+ * for the merged vector.  Buffers, hand-over, timeouts_dev, spin_limit and the bits of the result as for
  * llm_attn_decode_rope_oproj (the two entry points may share one ring of buffers); any position below max_pos.
  * Limits: Hq*hd <= 4096, N <= 24 * (CUs - Hq). */
 int llm_attn_long_oproj_supported(int n_heads, int n_kv_heads, int head_dim, int N); /* 1 or 0, current device */
@@ -225,7 +234,7 @@ int llm_attn_decode_rope_long_oproj(const uint16_t *qkv_dev, uint16_t *k_cache_d
                                     const int32_t *pos_dev, const float *table_dev, int n_heads, int n_kv_heads,
                                     int head_dim, int max_pos, void *workspace_dev, const uint16_t *w_dev,
                                     const uint16_t *residual_dev, uint16_t *out_dev, int N, int32_t *timeouts_dev,
-                                    llm_stream_t stream);
+                                    int spin_limit, llm_stream_t stream);
 /* The same step for `batch` (<= 16) independent sequences in one launch: row z of qkv_dev belongs to the
  * sequence with caches k_caches[z], v_caches[z] (host arrays of device pointers) at position positions[z];
  * workspace_dev holds batch * llm_attn_decode_workspace_bytes().  No counterpart in the reference (it
@@ -263,57 +272,6 @@ size_t llm_sample_candidates_head_bytes(int k);
 int llm_sample_candidates_max_vocab(void); /* larger vocabularies are rejected */
 int llm_sample_candidates(const uint16_t *logits_dev, const float *exp_table_dev, int vocab, int k,
                           void *out_dev, llm_stream_t stream);
-
-/* ---- measurement aid ---------------------------------------------------------------------------- */
-/* No counterpart in the reference.  Runs nothing but MFMAs on every CU for about ms_target milliseconds
- * and reports the sustained rate: kind 0 with constant operands, kind 1 with operands distributed like
- * the prompt pass's (N(0,1) activations, N(0,0.02) weights), both with v_mfma_f32_32x32x16_f16; kinds 2
- * and 3 the same with v_mfma_f32_16x16x32_f16.  The random-operand figures are the ceiling that the
- * power limit of the board leaves to the prompt-pass GEMMs. */
-int llm_mfma_probe(int kind, float ms_target, double *tflops, float *ms_out, llm_stream_t stream);
-
-/* ---- one decode token in one launch ------------------------------------------------------------- */
-/* Replaces, for positions below 512, the whole chain that inference() issues for one new token
- * (src/inference/inference.cu:149-193 at T = 1: embedding, 32 x {norm, QKV, RoPE, attention, O, +res,
- * norm, gate/up, down, +res}, final norm, LM head) except the final argmax reduction: one resident
- * workgroup per CU walks through all phases, the vectors between phases are handed over inside the
- * kernel.  Logits equal the per-kernel path (llm_norm_linear, llm_attn_decode_rope, llm_linear,
- * llm_norm_linear_swiglu, llm_norm_lmhead_argmax) bit for bit.
- * layers_dev: device array of n_layers llm_decode_layer (wqkv = the q, k, v matrices adjacent in memory).
- * ring_cur_dev / ring_next_dev: two hand-over buffer sets of llm_decode_fused_ring_halves() fp16 each,
- * both initialised once with llm_attn_oproj_buffer_init(); consecutive tokens alternate them (a launch
- * works in ring_cur and re-arms ring_next).  The token read is tokens_dev[*pos_dev]; K and V of the
- * token are appended to the caches at *pos_dev.  phase_begin/phase_end: 0 and llm_decode_fused_phases()
- * for the whole token (sub-ranges of phases 4*layer + {0 QKV, 1 attention + O, 2 gate/up, 3 down},
- * last = LM head, are for tests; they use the same ring_cur).  The LM-head phase leaves
- * llm_decode_fused_candidates() packed argmax candidates in candidates_dev: finish with
- * llm_argmax_finish().  timeouts_dev: one int32, zeroed by the caller, counts bounded waits that gave up
- * (must stay 0).  Launches that share buffers must not overlap; nothing else may occupy the GPU's CUs
- * for long while a launch runs (its workgroups wait for one another). */
-typedef struct {
-    const uint16_t *in_ln, *wqkv, *wo, *post_ln, *wgate, *wup, *wdown;
-    uint16_t *k_cache, *v_cache;
-} llm_decode_layer;
-typedef struct {
-    int n_layers, d_model, n_heads, n_kv_heads, head_dim, ffn_dim, vocab, max_pos;
-    double rms_eps;
-    const float *rope_table_dev;
-    const int32_t *pos_dev, *tokens_dev;
-    const uint16_t *embed_dev, *final_gain_dev, *lm_head_dev;
-    uint16_t *logits_dev;
-    void *candidates_dev;
-} llm_decode_desc;
-int llm_decode_fused_supported(const llm_decode_desc *desc); /* 1 or 0 on the current device */
-size_t llm_decode_fused_ring_halves(const llm_decode_desc *desc);
-int llm_decode_fused_candidates(const llm_decode_desc *desc);
-int llm_decode_fused_phases(const llm_decode_desc *desc);
-int llm_decode_fused(const llm_decode_desc *desc, const llm_decode_layer *layers_dev, uint16_t *ring_cur_dev,
-                     uint16_t *ring_next_dev, int phase_begin, int phase_end, int32_t *timeouts_dev,
-                     llm_stream_t stream);
-/* Final reduction over n packed candidates (as llm_norm_lmhead_argmax does after its GEMV): token_dev,
- * and tokens_dev[*pos_dev + 1] with *pos_dev incremented when tokens_dev/pos_dev are given. */
-int llm_argmax_finish(const void *candidates_dev, int n, int32_t *token_dev, int32_t *tokens_dev,
-                      int32_t *pos_dev, llm_stream_t stream);
 
 /* ---- LM head + argmax ------------------------------------------------------------ */
 /* Replaces compute_lm_head (src/inference/inference.cu:1003-1028) with the

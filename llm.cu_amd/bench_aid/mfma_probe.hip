@@ -72,47 +72,52 @@ template <bool SMALL> __global__ __launch_bounds__(256) void mfma_probe_kernel(f
 
 extern "C" {
 
-// Runs the probe for about `ms_target` milliseconds on `stream` and returns the sustained rate.
+// Runs the probe for about `ms_target` milliseconds on the default stream and returns the sustained rate.
 // kind: 0 constant operands, 1 random operands shaped like the prompt pass's (N(0,1) x N(0,0.02)), both with
-// v_mfma_f32_32x32x16_f16; 2 and 3: the same with v_mfma_f32_16x16x32_f16.
-int llm_mfma_probe(int kind, float ms_target, double *tflops, float *ms_out, llm_stream_t stream) {
-    LLM_REQUIRE(tflops && kind >= 0 && kind <= 3 && ms_target > 0.f, "llm_mfma_probe: arguments");
-    int cus = 0;
-    int rc = llm_cu_count_cached(&cus);
-    if (rc != LLM_OK) return rc;
+// v_mfma_f32_32x32x16_f16; 2 and 3: the same with v_mfma_f32_16x16x32_f16.  Returns 0, or the hipError_t of the
+// call that failed (1 for bad arguments).  Built into its own shared object (libllmcu_probe.so) that only
+// `bench.py --ceiling` loads; the token-loop library does not carry it.
+int mfma_probe(int kind, float ms_target, double *tflops, float *ms_out) {
+    if (!tflops || kind < 0 || kind > 3 || !(ms_target > 0.f)) return 1;
+    int dev = 0, cus = 0;
+    hipError_t err = hipGetDevice(&dev);
+    if (err == hipSuccess) err = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+    if (err != hipSuccess) return (int)err;
     float *sink = nullptr;
-    LLM_HIP_CHECK(hipMalloc((void **)&sink, 4));
-    hipEvent_t e0, e1;
-    LLM_HIP_CHECK(hipEventCreate(&e0));
-    LLM_HIP_CHECK(hipEventCreate(&e1));
-    hipStream_t s = (hipStream_t)stream;
+    hipEvent_t e0 = nullptr, e1 = nullptr;
     const int grid = cus * 2; // 8 wavefronts per CU, two per SIMD
-    auto run = [&](int iters, float *ms) -> int {
-        LLM_HIP_CHECK(hipEventRecord(e0, s));
-        if (kind & 2) mfma_probe_kernel<true><<<dim3(grid), dim3(256), 0, s>>>(sink, iters, kind);
-        else mfma_probe_kernel<false><<<dim3(grid), dim3(256), 0, s>>>(sink, iters, kind);
-        LLM_LAUNCH_CHECK("mfma_probe_kernel");
-        LLM_HIP_CHECK(hipEventRecord(e1, s));
-        LLM_HIP_CHECK(hipEventSynchronize(e1));
-        LLM_HIP_CHECK(hipEventElapsedTime(ms, e0, e1));
-        return LLM_OK;
+    auto run = [&](int iters, float *ms) -> hipError_t {
+        hipError_t e = hipEventRecord(e0, nullptr);
+        if (e != hipSuccess) return e;
+        if (kind & 2) mfma_probe_kernel<true><<<dim3(grid), dim3(256), 0, nullptr>>>(sink, iters, kind);
+        else mfma_probe_kernel<false><<<dim3(grid), dim3(256), 0, nullptr>>>(sink, iters, kind);
+        if ((e = hipGetLastError()) != hipSuccess) return e;
+        if ((e = hipEventRecord(e1, nullptr)) != hipSuccess) return e;
+        if ((e = hipEventSynchronize(e1)) != hipSuccess) return e;
+        return hipEventElapsedTime(ms, e0, e1);
     };
     float ms = 0.f;
     int iters = 10000;
-    rc = run(iters, &ms); // calibration (and warm-up)
-    if (rc != LLM_OK) return rc;
-    double want = (double)iters * ms_target / (ms > 0.01f ? ms : 0.01f);
-    if (want > 2.0e8) want = 2.0e8;
-    iters = want < 1000 ? 1000 : (int)want;
-    rc = run(iters, &ms);
-    if (rc != LLM_OK) return rc;
-    const double flops = (double)grid * 4 /*wavefronts*/ * iters * 16.0 * (2.0 * 32 * 32 * 16);
-    *tflops = flops / (ms * 1e-3) / 1e12;
-    if (ms_out) *ms_out = ms;
-    (void)hipEventDestroy(e0);
-    (void)hipEventDestroy(e1);
-    (void)hipFree(sink);
-    return LLM_OK;
+    err = hipMalloc((void **)&sink, 4);
+    if (err == hipSuccess) err = hipEventCreate(&e0);
+    if (err == hipSuccess) err = hipEventCreate(&e1);
+    if (err == hipSuccess) err = run(iters, &ms); // calibration (and warm-up)
+    if (err == hipSuccess) {
+        double want = (double)iters * ms_target / (ms > 0.01f ? ms : 0.01f);
+        if (want > 2.0e8) want = 2.0e8;
+        iters = want < 1000 ? 1000 : (int)want;
+        err = run(iters, &ms);
+    }
+    if (err == hipSuccess) {
+        const double flops = (double)grid * 4 /*wavefronts*/ * iters * 16.0 * (2.0 * 32 * 32 * 16);
+        *tflops = flops / (ms * 1e-3) / 1e12;
+        if (ms_out) *ms_out = ms;
+    }
+    // every path releases what it took
+    if (e0) (void)hipEventDestroy(e0);
+    if (e1) (void)hipEventDestroy(e1);
+    if (sink) (void)hipFree(sink);
+    return (int)err;
 }
 
 } // extern "C"

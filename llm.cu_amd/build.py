@@ -1,6 +1,8 @@
 """Builds libllmcu.so: the gfx950 kernels + C-ABI (csrc/*.hip, hipcc) and the
 reference-shaped host layer (src/**/*.cpp, g++) in one shared library, plus the
-`llama3_main` driver.  Everything lands in-tree next to this file.
+`llama3_main` driver and libllmcu_probe.so (bench_aid/mfma_probe.hip, the
+MFMA-only measurement aid that `bench.py --ceiling` loads; not part of the
+token-loop library).  Everything lands in-tree next to this file.
 
     python llm.cu_amd/build.py [--force] [-j N]
 """
@@ -18,6 +20,7 @@ INCLUDE = os.path.join(ROOT, "include")
 OBJ = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "libllmcu.so")
 MAIN = os.path.join(HERE, "llama3_main")
+PROBE_LIB = os.path.join(HERE, "libllmcu_probe.so")
 
 HIPCC = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
 HIP_FLAGS = [
@@ -78,6 +81,9 @@ def build(force=False, jobs=8, verbose=True):
         list(ex.map(_run, jobs_list))
     if force or jobs_list or not os.path.exists(LIB):
         _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs + ["-fopenmp", "-lm"])
+    probe_src = os.path.join(HERE, "bench_aid", "mfma_probe.hip")
+    if force or _newer([probe_src] + hip_hdr, PROBE_LIB):
+        _run([HIPCC] + HIP_FLAGS + ["-shared", probe_src, "-o", PROBE_LIB])
     main_src = os.path.join(HERE, "src", "main.cpp")
     if os.path.exists(main_src) and (force or _newer([main_src, LIB], MAIN)):
         _run([CXX] + CXX_FLAGS + [main_src, "-o", MAIN, "-L", HERE, "-lllmcu", "-Wl,-rpath,$ORIGIN"])

@@ -11,8 +11,7 @@ import os
 import numpy as np
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-# LLMCU_LIB names another build of the same library (kernel experiments side by side with the shipped build)
-LIB_PATH = os.environ.get("LLMCU_LIB") or os.path.join(HERE, "libllmcu.so")
+LIB_PATH = os.path.join(HERE, "libllmcu.so")
 
 LLM_OK, LLM_ERR_INVALID, LLM_ERR_HIP, LLM_ERR_NO_DEVICE = 0, 1, 2, 3
 
@@ -71,17 +70,6 @@ class CudaCache(C.Structure):
     ]
 
 
-class DecodeLayer(C.Structure):
-    _fields_ = [(k, C.c_void_p) for k in ("in_ln", "wqkv", "wo", "post_ln", "wgate", "wup", "wdown", "k_cache", "v_cache")]
-
-
-class DecodeDesc(C.Structure):
-    _fields_ = [(k, C.c_int) for k in ("n_layers", "d_model", "n_heads", "n_kv_heads", "head_dim", "ffn_dim", "vocab",
-                                       "max_pos")] + [("rms_eps", C.c_double)] + \
-        [(k, C.c_void_p) for k in ("rope_table_dev", "pos_dev", "tokens_dev", "embed_dev", "final_gain_dev", "lm_head_dev",
-                                   "logits_dev", "candidates_dev")]
-
-
 class GenStats(C.Structure):
     _fields_ = [("prefill_ms", C.c_double), ("decode_ms", C.c_double), ("n_prompt", C.c_int),
                 ("n_decode_steps", C.c_int)]
@@ -97,6 +85,7 @@ HIP_ABI = {
     "llm_device_cu_count": (_i, [C.POINTER(_i)]),
     "llm_malloc": (_i, [C.POINTER(_vp), _sz]),
     "llm_free": (_i, [_vp]),
+    "llm_mem_info": (_i, [C.POINTER(_sz), C.POINTER(_sz)]),
     "llm_malloc_host": (_i, [C.POINTER(_vp), _sz]),
     "llm_free_host": (_i, [_vp]),
     "llm_memcpy_h2d": (_i, [_vp, _vp, _sz, _vp]),
@@ -132,27 +121,20 @@ HIP_ABI = {
     "llm_attn_decode_rope_batch": (_i, [_vp, _i, _vp, _vp, _vp, _i, _vp, _i, _vp, _i, _i, _i, _i, _vp, _vp]),
     "llm_attn_oproj_supported": (_i, [_i, _i, _i, _i]),
     "llm_attn_oproj_buffer_init": (_i, [_vp, _i, _vp]),
-    "llm_attn_decode_rope_oproj": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _vp, _vp, _vp, _i, _vp, _vp]),
+    "llm_attn_decode_rope_oproj": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _vp, _vp, _vp, _i, _vp, _i, _vp]),
     "llm_sample_candidates_bytes": (_sz, [_i, _i]),
     "llm_sample_candidates_head_bytes": (_sz, [_i]),
     "llm_sample_candidates_max_vocab": (_i, []),
     "llm_sample_candidates": (_i, [_vp, _vp, _i, _i, _vp, _vp]),
     "llm_attn_decode_rope_long": (_i, [_vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _vp, _vp]),
     "llm_attn_long_oproj_supported": (_i, [_i, _i, _i, _i]),
-    "llm_attn_decode_rope_long_oproj": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _i, _vp, _vp]),
+    "llm_attn_decode_rope_long_oproj": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _i, _vp, _i, _vp]),
     "llm_norm_lmhead_argmax": (_i, [_vp, _vp, C.c_double, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp, _vp]),
     "llm_attn_decode_workspace_bytes": (_sz, [_i, _i]),
     "llm_attn_decode": (_i, [_vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _i, _vp, _vp]),
     "llm_attn_decode_noalloc_max_bytes": (_sz, []),
     "llm_attn_decode_noalloc": (_i, [_vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _i, _vp]),
     "llm_attn_prefill": (_i, [_vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp]),
-    "llm_mfma_probe": (_i, [_i, C.c_float, C.POINTER(C.c_double), C.POINTER(C.c_float), _vp]),
-    "llm_decode_fused_supported": (_i, [C.POINTER(DecodeDesc)]),
-    "llm_decode_fused_ring_halves": (_sz, [C.POINTER(DecodeDesc)]),
-    "llm_decode_fused_candidates": (_i, [C.POINTER(DecodeDesc)]),
-    "llm_decode_fused_phases": (_i, [C.POINTER(DecodeDesc)]),
-    "llm_decode_fused": (_i, [C.POINTER(DecodeDesc), _vp, _vp, _vp, _i, _i, _vp, _vp]),
-    "llm_argmax_finish": (_i, [_vp, _i, _vp, _vp, _vp, _vp]),
     "llm_lmhead_workspace_bytes": (_sz, [_i]),
     "llm_lmhead_argmax": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp, _vp]),
     "llm_argmax_f16": (_i, [_vp, _i, _vp, _vp, _vp]),
@@ -184,6 +166,9 @@ HOST_ABI = {
     "llama3_read_logits": (None, [_CP, _vp]),
     "llama3_set_hidden_inject": (None, [_CP, _vp]),
     "llama3_set_use_graph": (None, [_CP, _i]),
+    "llama3_set_handover": (None, [_CP, _i, _i]),
+    "llama3_handover_stats": (None, [_CP, C.POINTER(C.c_long), C.POINTER(C.c_long), C.POINTER(_i)]),
+    "llama3_test_mark_handover_timeout": (None, [_CP]),
     "llama3_set_error_handler": (None, [_vp]),
     "seeded_normal_bf16": (None, [_u64, _u64, _sz, C.c_float, _vp]),
     "seeded_tokens": (None, [_u64, _i, _i, _vp]),
@@ -214,9 +199,6 @@ HOST_ABI = {
     "llama3_set_device_sampling": (None, [_CP, _i]),
     "llama3_sampler_draw_counts": (None, [_CP, C.POINTER(C.c_long), C.POINTER(C.c_long)]),
     "llama3_sample_device_logits": (_i, [_CP, _vp]),
-    "llama3_set_fused_decode": (None, [_CP, _i]),
-    "llama3_fused_decode_active": (_i, [_CP]),
-    "llama3_read_fused_vectors": (None, [_CP, _i, _vp]),
     "llama3_cache_sampler_config": (None, [_CP, C.c_float, _i, C.c_float]),
     "llama3_sample_with": (_i, [_i, C.c_float, _i, C.c_float, _vp, _vp]),
 }

@@ -70,8 +70,11 @@ __global__ __launch_bounds__(AD_THREADS) void attn_decode_kernel(const AdArgs a)
 // host passes a ring of at least two buffers), so every launch finds its own buffer empty.
 // One workgroup per CU at most (grid <= number of CUs), and workgroups are dispatched in id order, so the
 // attention workgroups are running before any projection workgroup can wait for them: the wait cannot
-// deadlock.  It is bounded anyway (AO_SPIN_LIMIT rounds, after which the workgroup carries on and counts
-// a timeout in *timeouts for the host to see).
+// deadlock, also when launches of several streams share the device (each queue hands out its workgroups in
+// id order, so a resident projection workgroup implies that its launch's attention workgroups were handed
+// out before it).  It is bounded anyway (spin_limit rounds, AO_SPIN_LIMIT by default, after which the workgroup
+// carries on with whatever the buffer holds and counts a timeout in *timeouts: the host must then treat the
+// projection's output as invalid and redo the step).
 // ---------------------------------------------------------------------------
 #define AO_WAVES 8          // = AD_WAVES: both roles use 512 threads
 #define AO_ROWS 3           // weight rows per wavefront of the projection part, at most
@@ -87,7 +90,8 @@ struct AoArgs {
     int N, K;
     int n_owg;         // projection workgroups
     int rows;          // weight rows per wavefront (<= AO_ROWS)
-    int *timeouts;     // diagnostic: waits that ran into AO_SPIN_LIMIT
+    int *timeouts;     // waits that ran into the limit
+    int spin_limit;    // polling rounds before a wait gives up
 };
 
 // The projection role of a launch whose first n_first workgroups produce the projection's input vector (a.out,
@@ -107,10 +111,7 @@ __device__ __forceinline__ void ao_projection_part(const AdArgs &a, const AoArgs
     half_t resv[AO_ROWS];
     // a head start of a little under a microsecond for the attention's own loads (measured per launch: 12.2 -> 11.4 us
     // with the first version of the attention; against the current one three pauses beat 0-2 and 4-8)
-#ifndef AO_HEAD_START
-#define AO_HEAD_START 3
-#endif
-    for (int dl = 0; dl < AO_HEAD_START; ++dl) __builtin_amdgcn_s_sleep(8);
+    for (int dl = 0; dl < 3; ++dl) __builtin_amdgcn_s_sleep(8);
 #pragma unroll
     for (int r = 0; r < AO_ROWS; ++r) {
         int row = wslot + wtotal * r;
@@ -141,7 +142,7 @@ __device__ __forceinline__ void ao_projection_part(const AdArgs &a, const AoArgs
 #pragma unroll
             for (int i = 0; i < WPT; ++i) empty |= (v[i] & 0xFFFFu) == AO_EMPTY || (v[i] >> 16) == AO_EMPTY;
             if (!empty) break;
-            if (++spins > AO_SPIN_LIMIT) {
+            if (++spins > o.spin_limit) {
                 atomicAdd(o.timeouts, 1);
                 break;
             }
@@ -188,7 +189,7 @@ __global__ __launch_bounds__(AD_THREADS) void attn_oproj_kernel(const int32_t *p
                                                                 half_t *vc, const float *table, const half_t *w,
                                                                 int pos_host, int kvh_maxpos, half_t *attn_out,
                                                                 const half_t *res, half_t *out, uint16_t *next, int N,
-                                                                int K, int n_owg, int rows, int *timeouts) {
+                                                                int K, int n_owg, int rows, int *timeouts, int spin_limit) {
     AdArgs a = {};
     a.q = qkv;
     a.kc = kc;
@@ -200,7 +201,7 @@ __global__ __launch_bounds__(AD_THREADS) void attn_oproj_kernel(const int32_t *p
     a.n_kv_heads = kvh_maxpos & 0xff;
     a.max_pos = (int)((unsigned)kvh_maxpos >> 8);
     a.splits = 1;
-    const AoArgs o = {w, res, out, next, N, K, n_owg, rows, timeouts};
+    const AoArgs o = {w, res, out, next, N, K, n_owg, rows, timeouts, spin_limit};
     __shared__ float sc[G * AD_LS];
     __shared__ __attribute__((aligned(16))) half_t qs[G * HD];
     __shared__ __attribute__((aligned(16))) half_t knew[HD];
@@ -248,7 +249,7 @@ static int launch_attn_oproj(AdArgs a, AoArgs o, hipStream_t s) {
                 a.max_pos);
     attn_oproj_kernel<HD, G, DSN><<<dim3(n_attn + owg), dim3(AD_THREADS), 0, s>>>(
         a.pos_dev, a.q, a.kc, a.vc, a.table, o.w, a.pos_host, a.n_kv_heads | (a.max_pos << 8), a.out, o.res, o.out, o.next, o.N,
-        o.K, o.n_owg, o.rows, o.timeouts);
+        o.K, o.n_owg, o.rows, o.timeouts, o.spin_limit);
     LLM_LAUNCH_CHECK("attn_oproj_kernel");
     return LLM_OK;
 }
@@ -330,7 +331,7 @@ __global__ __launch_bounds__(AD_THREADS) void attn_span_kernel(const int32_t *po
     const int y = blockIdx.y;
     if (y >= n_active) return;
     attn_decode_body<HD, G, FUSED, HD, AD_LONG_LS_MAX, true>(a, sc, qs, knew, vnew, s_m, s_l, &s_last, pos, n_active, y, 0,
-                                                             y == n_active - 1, -1, nullptr, nullptr, span_len);
+                                                             y == n_active - 1, -1, span_len);
 }
 
 // AGENT_OUT: the head's result leaves as 8-byte device-scope stores with the "not written yet" pattern avoided,
@@ -469,7 +470,7 @@ __global__ __launch_bounds__(AD_THREADS) void merge_oproj_kernel(const int32_t *
                                                                  const float *ws_acc, const half_t *w, int pos_host,
                                                                  int kvh_maxpos, int splits_target, int N, int K, int n_owg,
                                                                  half_t *attn_out, const half_t *res, half_t *out,
-                                                                 uint16_t *next, int rows, int *timeouts) {
+                                                                 uint16_t *next, int rows, int *timeouts, int spin_limit) {
     AdArgs a = {};
     a.out = attn_out;
     a.pos_host = pos_host;
@@ -480,7 +481,7 @@ __global__ __launch_bounds__(AD_THREADS) void merge_oproj_kernel(const int32_t *
     a.span_target = (int)((unsigned)splits_target >> 16);
     a.ws_acc = const_cast<float *>(ws_acc);
     a.ws_ml = const_cast<float *>(ws_ml);
-    const AoArgs o = {w, res, out, next, N, K, n_owg, rows, timeouts};
+    const AoArgs o = {w, res, out, next, N, K, n_owg, rows, timeouts, spin_limit};
     static_assert(AD_MERGE_THREADS == AD_THREADS, "both roles share the workgroup size");
     __shared__ __attribute__((aligned(16))) half_t xs[AO_KSTEPS * 512];
     const int n_first = a.n_kv_heads * G;
@@ -525,7 +526,7 @@ static int launch_long_oproj(AdArgs a, AoArgs o, void *ws, hipStream_t s) {
     LLM_LAUNCH_CHECK("attn_span_kernel");
     merge_oproj_kernel<HD, G><<<dim3(Hq + o.n_owg), dim3(AD_THREADS), 0, s>>>(
         a.pos_dev, a.ws_ml, a.ws_acc, o.w, a.pos_host, a.n_kv_heads | (a.max_pos << 8), a.splits | (a.span_target << 16), o.N, o.K,
-        o.n_owg, a.out, o.res, o.out, o.next, o.rows, o.timeouts);
+        o.n_owg, a.out, o.res, o.out, o.next, o.rows, o.timeouts, o.spin_limit);
     LLM_LAUNCH_CHECK("merge_oproj_kernel");
     return LLM_OK;
 }
@@ -590,7 +591,7 @@ __global__ __launch_bounds__(AD_THREADS) void attn_span_batch_kernel(const AdArg
     const int y = blockIdx.y;
     if (y >= n_active) return;
     attn_decode_body<HD, G, true, HD, AD_LONG_LS_MAX, true>(a, sc, qs, knew, vnew, s_m, s_l, &s_last, a.pos_host, n_active,
-                                                            y, 0, y == n_active - 1, -1, nullptr, nullptr, span_len);
+                                                            y, 0, y == n_active - 1, -1, span_len);
 }
 
 template <int HD, int G>
@@ -656,14 +657,27 @@ size_t llm_attn_decode_workspace_bytes(int n_heads, int head_dim) {
     return sizeof(float) * (size_t)n_heads * AD_MAX_SPLITS * (head_dim + 2) + sizeof(int) * (size_t)n_heads;
 }
 
+// what llm_attn_decode and llm_attn_decode_noalloc require of their arguments, checked before either launches anything
+static int attn_decode_check(const void *q, const void *kc, const void *vc, const void *out, int ctx_host,
+                             const int32_t *ctx_dev, int n_heads, int n_kv_heads, int head_dim, int max_pos) {
+    LLM_REQUIRE(q && kc && vc && out, "llm_attn_decode: null pointer");
+    LLM_REQUIRE(n_kv_heads > 0 && n_heads > 0 && n_heads % n_kv_heads == 0, "llm_attn_decode: heads %d/%d", n_heads, n_kv_heads);
+    LLM_REQUIRE(max_pos > 0 && max_pos % 64 == 0, "llm_attn_decode: max_pos=%d must be a multiple of 64", max_pos);
+    LLM_REQUIRE((max_pos + AD_LS - 1) / AD_LS <= AD_MAX_SPLITS, "llm_attn_decode: max_pos=%d exceeds %d", max_pos, AD_MAX_SPLITS * AD_LS);
+    LLM_REQUIRE(ctx_dev || (ctx_host >= 1 && ctx_host <= max_pos), "llm_attn_decode: ctx=%d of %d", ctx_host, max_pos);
+    LLM_REQUIRE(aligned16(q) && aligned16(kc) && aligned16(vc), "llm_attn_decode: pointers must be 16-byte aligned");
+    const int G = n_heads / n_kv_heads;
+    const bool built = (head_dim == 128 && (G == 1 || G == 4 || G == 8)) || ((head_dim == 64 || head_dim == 32) && (G == 1 || G == 4));
+    LLM_REQUIRE(built, "llm_attn_decode: head_dim=%d with group size %d is not built", head_dim, G);
+    return LLM_OK;
+}
+
 int llm_attn_decode(const uint16_t *q, const uint16_t *kc, const uint16_t *vc, uint16_t *out, int ctx_host,
                     const int32_t *ctx_dev, int n_heads, int n_kv_heads, int head_dim, int max_pos, void *workspace,
                     llm_stream_t stream) {
-    LLM_REQUIRE(q && kc && vc && out && workspace, "llm_attn_decode: null pointer");
-    LLM_REQUIRE(n_kv_heads > 0 && n_heads % n_kv_heads == 0, "llm_attn_decode: heads %d/%d", n_heads, n_kv_heads);
-    LLM_REQUIRE(max_pos > 0 && max_pos % 64 == 0, "llm_attn_decode: max_pos=%d must be a multiple of 64", max_pos);
-    LLM_REQUIRE(ctx_dev || (ctx_host >= 1 && ctx_host <= max_pos), "llm_attn_decode: ctx=%d of %d", ctx_host, max_pos);
-    LLM_REQUIRE(aligned16(q) && aligned16(kc) && aligned16(vc), "llm_attn_decode: pointers must be 16-byte aligned");
+    LLM_REQUIRE(workspace, "llm_attn_decode: null workspace");
+    int rc = attn_decode_check(q, kc, vc, out, ctx_host, ctx_dev, n_heads, n_kv_heads, head_dim, max_pos);
+    if (rc != LLM_OK) return rc;
     AdArgs a = {};
     a.q = (const half_t *)q;
     a.kc = (half_t *)kc;
@@ -722,10 +736,13 @@ int llm_attn_decode_noalloc(const uint16_t *q, const uint16_t *kc, const uint16_
                 "llm_attn_decode_noalloc: %d heads of %d dims need %zu scratch bytes; the built-in scratch holds %zu "
                 "(at most %d heads of at most %d dims): use llm_attn_decode with a workspace",
                 n_heads, head_dim, need, (size_t)AD_STATIC_BYTES, AD_STATIC_MAX_HEADS, AD_STATIC_MAX_HEAD_DIM);
+    // every argument is checked before the first launch: an invalid call enqueues nothing
+    int rc = attn_decode_check(q, kc, vc, out, ctx_host, ctx_dev, n_heads, n_kv_heads, head_dim, max_pos);
+    if (rc != LLM_OK) return rc;
     int device = 0;
     LLM_HIP_CHECK(hipGetDevice(&device));
     void *ws = nullptr;
-    int rc = scratch_for_device(device, &ws);
+    rc = scratch_for_device(device, &ws);
     if (rc != LLM_OK) return rc;
     // The array keeps what the last call left, and the counters sit behind the partial results at an
     // offset that depends on (n_heads, head_dim): after a call with another shape that spot holds
@@ -761,7 +778,7 @@ int llm_attn_decode_rope(const uint16_t *qkv, uint16_t *kc, uint16_t *vc, uint16
 int llm_attn_decode_rope_oproj(const uint16_t *qkv, uint16_t *kc, uint16_t *vc, uint16_t *attn_out, uint16_t *attn_out_next,
                                int pos_host, const int32_t *pos_dev, const float *table, int n_heads, int n_kv_heads,
                                int head_dim, int max_pos, const uint16_t *w, const uint16_t *residual, uint16_t *out, int N,
-                               int32_t *timeouts_dev, llm_stream_t stream) {
+                               int32_t *timeouts_dev, int spin_limit, llm_stream_t stream) {
     LLM_REQUIRE(qkv && kc && vc && attn_out && attn_out_next && table && w && out && timeouts_dev,
                 "llm_attn_decode_rope_oproj: null pointer");
     LLM_REQUIRE(attn_out != attn_out_next, "llm_attn_decode_rope_oproj: a launch cannot refill its own buffer");
@@ -793,6 +810,7 @@ int llm_attn_decode_rope_oproj(const uint16_t *qkv, uint16_t *kc, uint16_t *vc, 
     o.N = N;
     o.K = K;
     o.timeouts = timeouts_dev;
+    o.spin_limit = spin_limit >= 0 ? spin_limit : AO_SPIN_LIMIT;
     hipStream_t s = (hipStream_t)stream;
     const int G = n_heads / n_kv_heads;
 #define AO_CASE(HD_, G_) \
@@ -874,7 +892,7 @@ int llm_attn_decode_rope_long_oproj(const uint16_t *qkv, uint16_t *kc, uint16_t 
                                     uint16_t *attn_out_next, int pos_host, const int32_t *pos_dev, const float *table,
                                     int n_heads, int n_kv_heads, int head_dim, int max_pos, void *workspace,
                                     const uint16_t *w, const uint16_t *residual, uint16_t *out, int N,
-                                    int32_t *timeouts_dev, llm_stream_t stream) {
+                                    int32_t *timeouts_dev, int spin_limit, llm_stream_t stream) {
     LLM_REQUIRE(qkv && kc && vc && attn_out && attn_out_next && table && workspace && w && out && timeouts_dev,
                 "llm_attn_decode_rope_long_oproj: null pointer");
     LLM_REQUIRE(attn_out != attn_out_next, "llm_attn_decode_rope_long_oproj: a launch cannot refill its own buffer");
@@ -906,6 +924,7 @@ int llm_attn_decode_rope_long_oproj(const uint16_t *qkv, uint16_t *kc, uint16_t 
     o.N = N;
     o.K = K;
     o.timeouts = timeouts_dev;
+    o.spin_limit = spin_limit >= 0 ? spin_limit : AO_SPIN_LIMIT;
     hipStream_t s = (hipStream_t)stream;
     const int G = n_heads / n_kv_heads;
 #define AO_CASE(HD_, G_) \

@@ -46,13 +46,6 @@ __host__ __device__ inline int ad_long_spans(int ctx, int target) {
 // that write.
 //
 // NDIM is the number of head dims this workgroup produces, LS the span length.
-// POLL_IN (with FUSED): a.q is a hand-over buffer that other workgroups of the same kernel are still
-// filling: its words are read at device scope until none holds AD_EMPTY16 (the pattern the buffer was
-// armed with, never written as a value) and staged in qkv_l ([(G + 2) * HD]: the group's queries, the new
-// key, the new value).  The wait is bounded: after AD_POLL_LIMIT rounds *timeouts is incremented and the
-// workgroup carries on.
-#define AD_EMPTY16 0xFFFFu
-#define AD_POLL_LIMIT (1 << 18)
 
 // LDS of the attention.  The K staging buffer depends on the head size only: a kernel that instantiates the body
 // twice (for a quarter of the dims and for all of them) holds it once.
@@ -81,12 +74,11 @@ template <int G> __device__ __forceinline__ float *ad_lds_ml() {
 // Every cache-row load is issued unconditionally (positions beyond the span re-read its last row and are masked
 // afterwards): with a fixed number of loads in flight the waits can name the loads they need, and the rotation
 // of the new token, whose inputs are requested first, runs while the cache rows are still on their way.
-template <int HD, int G, bool FUSED, int NDIM, int LS, bool TWOPASS, bool AGENT_OUT, bool POLL_IN, int NB>
+template <int HD, int G, bool FUSED, int NDIM, int LS, bool TWOPASS, bool AGENT_OUT, int NB>
 __device__ __forceinline__ void attn_decode_span(const AdArgs &a, half_t *qs, half_t *knew, half_t *vnew,
                                                  half_t *kst_all, float *ow_all, float *ml_all, const int pos,
                                                  const int n_active, const int split, const int d_begin,
-                                                 const bool appender, const int kvh, half_t *qkv_l, int *timeouts,
-                                                 const int span_len) {
+                                                 const bool appender, const int kvh, const int span_len) {
     constexpr int LPP = HD / 8;   // lanes per K row
     constexpr int PPW = 64 / LPP; // K rows per load instruction of a wavefront
     constexpr int NPB = 32 / PPW; // load instructions per block
@@ -113,12 +105,11 @@ __device__ __forceinline__ void attn_decode_span(const AdArgs &a, half_t *qs, ha
     // ---- 0. the new token's inputs, requested before the cache rows -----------------------
     constexpr int NRI = ((G + 1) * HALF + AD_THREADS - 1) / AD_THREADS; // rotation pairs per thread
     constexpr int NVI = (HD + AD_THREADS - 1) / AD_THREADS;             // new-v elements per thread
-    constexpr bool EARLY = FUSED && !POLL_IN;
     uint32_t pair_r[NRI];
     float2_t cs_r[NRI];
     half_t vnew_r[NVI];
     half8_t q_r = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
-    if (EARLY) {
+    if (FUSED) {
         const int Hq = a.n_kv_heads * G;
         const float *cs = a.table + (size_t)pos * HALF * 2;
 #pragma unroll
@@ -167,44 +158,13 @@ __device__ __forceinline__ void attn_decode_span(const AdArgs &a, half_t *qs, ha
 
     // ---- 2. queries into LDS; fused: rotate them and the new K, append K/V ---------
     if (FUSED) {
-        const int Hq = a.n_kv_heads * G;
-        const half_t *qkv = a.q;
-        const float *cs = a.table + (size_t)pos * HALF * 2;
-        if (POLL_IN) {
-            constexpr int NQ = G * HD / 2, NK = HD / 2; // 32-bit words
-            const uint32_t *base = reinterpret_cast<const uint32_t *>(qkv);
-            int spins = 0;
-            for (int wi = tid; wi < NQ + 2 * NK; wi += AD_THREADS) {
-                const size_t sw = wi < NQ        ? (size_t)kvh * G * HD / 2 + wi
-                                  : wi < NQ + NK ? ((size_t)Hq * HD + (size_t)kvh * HD) / 2 + (wi - NQ)
-                                                 : ((size_t)(Hq + a.n_kv_heads) * HD + (size_t)kvh * HD) / 2 + (wi - NQ - NK);
-                uint32_t v;
-                for (;;) {
-                    v = __hip_atomic_load(base + sw, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                    if ((v & 0xFFFFu) != AD_EMPTY16 && (v >> 16) != AD_EMPTY16) break;
-                    if (++spins > AD_POLL_LIMIT) {
-                        if (timeouts) atomicAdd(timeouts, 1);
-                        break;
-                    }
-                    __builtin_amdgcn_s_sleep(8); // a few hundred cycles: the pollers must not crowd the producers' memory traffic
-                }
-                reinterpret_cast<uint32_t *>(qkv_l)[wi] = v;
-            }
-            __syncthreads();
-        }
 #pragma unroll
         for (int r = 0; r < NRI; ++r) {
             const int p = tid + r * AD_THREADS;
             if (p < (G + 1) * HALF) {
                 const int h = p / HALF, i = p % HALF; // h == G: the new key
-                float c, sn, e, o;
-                if (EARLY) {
-                    const half2_t pr = __builtin_bit_cast(half2_t, pair_r[r]);
-                    c = cs_r[r][0], sn = cs_r[r][1], e = (float)pr[0], o = (float)pr[1];
-                } else {
-                    const half_t *src = qkv_l + (size_t)h * HD + 2 * i;
-                    c = cs[2 * i], sn = cs[2 * i + 1], e = (float)src[0], o = (float)src[1];
-                }
+                const half2_t pr = __builtin_bit_cast(half2_t, pair_r[r]);
+                const float c = cs_r[r][0], sn = cs_r[r][1], e = (float)pr[0], o = (float)pr[1];
                 const float ce = c * e, so = sn * o, se = sn * e, co = c * o;
                 const half_t re = (half_t)(ce - so), ro = (half_t)(se + co);
                 if (h < G) {
@@ -224,7 +184,7 @@ __device__ __forceinline__ void attn_decode_span(const AdArgs &a, half_t *qs, ha
         for (int r = 0; r < NVI; ++r) {
             const int d = tid + r * AD_THREADS;
             if (d < HD) {
-                const half_t v = EARLY ? vnew_r[r] : qkv_l[(size_t)(G + 1) * HD + d];
+                const half_t v = vnew_r[r];
                 vnew[d] = v;
                 if (appender) vrow0[(size_t)d * max_pos + pos] = v;
             }
@@ -369,12 +329,11 @@ __device__ __forceinline__ void attn_decode_span(const AdArgs &a, half_t *qs, ha
     }
 }
 
-template <int HD, int G, bool FUSED, int NDIM, int LS, bool TWOPASS = false, bool AGENT_OUT = false, bool POLL_IN = false>
+template <int HD, int G, bool FUSED, int NDIM, int LS, bool TWOPASS = false, bool AGENT_OUT = false>
 __device__ __forceinline__ void attn_decode_body(const AdArgs &a, float *sc, half_t *qs, half_t *knew, half_t *vnew,
                                                  float *s_m, float *s_l, int *s_last, const int pos,
                                                  const int n_active, const int split, const int d_begin,
-                                                 const bool appender, const int kvh_arg = -1, half_t *qkv_l = nullptr,
-                                                 int *timeouts = nullptr, const int span_len_arg = 0) {
+                                                 const bool appender, const int kvh_arg = -1, const int span_len_arg = 0) {
     static_assert(LS == 256 || LS == 512, "span length");
     const int span_len = span_len_arg > 0 ? span_len_arg : LS; // positions per span (a multiple of 8, at most LS)
     (void)s_m; // the statistics of a span live in ad_lds_ml; s_l and sc serve the merge of several spans below
@@ -385,11 +344,11 @@ __device__ __forceinline__ void attn_decode_body(const AdArgs &a, float *sc, hal
     const int tid = threadIdx.x;
     // one or two blocks per wavefront, each form with its own fixed number of loads in flight
     if (LS == 512 && pos + 1 - split * span_len > 256 && span_len > 256)
-        attn_decode_span<HD, G, FUSED, NDIM, LS, TWOPASS, AGENT_OUT, POLL_IN, LS / 256>(
-            a, qs, knew, vnew, kst_all, ow_all, ml_all, pos, n_active, split, d_begin, appender, kvh, qkv_l, timeouts, span_len);
+        attn_decode_span<HD, G, FUSED, NDIM, LS, TWOPASS, AGENT_OUT, LS / 256>(
+            a, qs, knew, vnew, kst_all, ow_all, ml_all, pos, n_active, split, d_begin, appender, kvh, span_len);
     else
-        attn_decode_span<HD, G, FUSED, NDIM, LS, TWOPASS, AGENT_OUT, POLL_IN, 1>(
-            a, qs, knew, vnew, kst_all, ow_all, ml_all, pos, n_active, split, d_begin, appender, kvh, qkv_l, timeouts, span_len);
+        attn_decode_span<HD, G, FUSED, NDIM, LS, TWOPASS, AGENT_OUT, 1>(
+            a, qs, knew, vnew, kst_all, ow_all, ml_all, pos, n_active, split, d_begin, appender, kvh, span_len);
     if (n_active == 1 && !TWOPASS) return;
     if (TWOPASS) return; // attn_merge_kernel combines the spans
 

@@ -35,9 +35,7 @@
 
 #define AP_BQ 32
 #define AP_BKEY 64
-#ifndef AP_PIPE_MIN_ROWS
 #define AP_PIPE_MIN_ROWS 64 // shorter blocks of rows take attn_prefill_kernel
-#endif
 
 // Workgroup = one KV head x AP_QT query tiles (2, or 1 for groups of 8 heads); wavefront w serves query head
 // kvh*G + w%G on tile w/G, so G*AP_QT wavefronts share every K/V tile.  K/V

@@ -311,10 +311,8 @@ int llm_rmsnorm(const uint16_t *x, const uint16_t *gain, uint16_t *y, int T, int
     if (T == 0) return LLM_OK;
     hipStream_t s = (hipStream_t)stream;
     const int n = d / 4;
-#ifndef RMS_ROW_THREADS
-#define RMS_ROW_THREADS 128
-#endif
-    if (n >= 256 && n <= RMS_ROW_THREADS * RMS_MAX_R && RMS_ROW_THREADS < 256) {
+    constexpr int RMS_ROW_THREADS = 128;
+    if (n >= 256 && n <= RMS_ROW_THREADS * RMS_MAX_R) {
         rmsnorm_kernel<RMS_ROW_THREADS><<<dim3(T), dim3(RMS_ROW_THREADS), 0, s>>>((const half_t *)x, (const half_t *)gain, (half_t *)y, d, eps);
     } else if (n >= 256) {
         rmsnorm_kernel<256><<<dim3(T), dim3(256), 0, s>>>((const half_t *)x, (const half_t *)gain, (half_t *)y, d, eps);

@@ -358,10 +358,7 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_kernel(const half_t *__res
         const int per = nblk / 8;
         if (per > 0 && bid < per * 8) bid = (bid % 8) * per + bid / 8;
     }
-#ifndef GEMM_GROUP_M
-#define GEMM_GROUP_M 8
-#endif
-    constexpr int GROUP_M = GEMM_GROUP_M;
+    constexpr int GROUP_M = 8;
     const int group = bid / (GROUP_M * tiles_n);
     const int first_m = group * GROUP_M;
     const int gsz = tiles_m - first_m < GROUP_M ? tiles_m - first_m : GROUP_M;
@@ -746,9 +743,6 @@ __global__ __launch_bounds__(WGM * WGN * 64, OCC) void gemm_dma_kernel(const hal
 // activation and 8 weight fragments each, read during the sub-step before); the workgroup barrier sits between
 // the two: by then every wave has read the last fragments of the current stage and the next tile (issued
 // during the previous step's second sub-step, one load behind every fourth MFMA) must have landed.
-#ifndef DMA64_WIDE_EPILOGUE
-#define DMA64_WIDE_EPILOGUE 1 // 0: keep the 8-byte stores (for timing the two forms side by side)
-#endif
 template <int NB>
 __global__ __launch_bounds__(256, 1) void gemm_dma64_kernel(const half_t *__restrict__ x, int ldx, const half_t *__restrict__ w,
                                                            const half_t *__restrict__ w2, const half_t *res, int ldr,
@@ -896,7 +890,7 @@ __global__ __launch_bounds__(256, 1) void gemm_dma64_kernel(const half_t *__rest
     // results of two neighbouring weight blocks (v_permlane16_swap), after which a lane holds eight consecutive
     // columns: 16-byte stores and residual loads that cover 64 contiguous bytes of a row per instruction instead
     // of 8-byte ones that cover 32.  Same values, same roundings.
-    const bool wide = DMA64_WIDE_EPILOGUE && ((uintptr_t)out & 15u) == 0 && ldo % 8 == 0 && N % 8 == 0 &&
+    const bool wide = ((uintptr_t)out & 15u) == 0 && ldo % 8 == 0 && N % 8 == 0 &&
                       (!(NB == 1 && res) || (((uintptr_t)res & 15u) == 0 && ldr % 8 == 0));
     if (wide) {
         const int g = lane / 16;

@@ -57,10 +57,7 @@ __global__ __launch_bounds__(GEMV_THREADS) void gemv_kernel(const half_t *x, con
                         ids,   ids_offset, x_copy, vocab};
     constexpr int NW = MODE == GV_SWIGLU ? 2 : 1; // weight streams per row
     constexpr bool PLAIN = MODE == GV_PLAIN || MODE == GV_EMBED;
-#ifndef GEMV_NBUF1
-#define GEMV_NBUF1 2
-#endif
-    constexpr int NBUF = NW == 2 ? 2 : GEMV_NBUF1; // steps in flight per wavefront (2 KB per stream and step)
+    constexpr int NBUF = 2; // steps in flight per wavefront (2 KB per stream and step)
     extern __shared__ __attribute__((aligned(16))) half_t xs[];
     __shared__ float red[GEMV_THREADS + 1];
     __shared__ unsigned long long best[GEMV_WAVES];
@@ -101,9 +98,7 @@ __global__ __launch_bounds__(GEMV_THREADS) void gemv_kernel(const half_t *x, con
     // the activation loads go out first, then NBUF steps of weights; only then
     // does anything wait (the norm's reduction), so HBM is busy throughout
     RmsRow<GEMV_NORM_R> xr;
-#ifndef GEMV_XRAW
-#define GEMV_XRAW 8
-#endif
+    constexpr int GEMV_XRAW = 8;
     half8_t xraw[GEMV_XRAW]; // the first GEMV_XRAW * 2048 elements of a plain input vector, asked for before the weights
     if (MODE == GV_EMBED) {
         // the weights do not depend on the token: they go out first, the two dependent loads of the id (position,
@@ -283,14 +278,8 @@ __global__ __launch_bounds__(1024) void argmax_final_kernel(const unsigned long 
 // the norm-fused QKV projection and the 128K-row LM head amortise their
 // per-workgroup prologue over more than one row.
 static int rows_per_wave(int mode, int N, bool norm) {
-#ifndef GEMV_RPW_LM
-#define GEMV_RPW_LM 3
-#endif
-#ifndef GEMV_RPW_QKV
-#define GEMV_RPW_QKV 2
-#endif
-    if (mode == GV_LMHEAD) return N >= 32768 ? GEMV_RPW_LM : 1;
-    if ((mode == GV_PLAIN || mode == GV_EMBED) && norm && N >= 6144) return GEMV_RPW_QKV;
+    if (mode == GV_LMHEAD) return N >= 32768 ? 3 : 1;
+    if ((mode == GV_PLAIN || mode == GV_EMBED) && norm && N >= 6144) return 2;
     return 1;
 }
 
@@ -352,15 +341,6 @@ int llm_norm_lmhead_argmax(const uint16_t *x, const uint16_t *gain, double eps, 
     if (rc != LLM_OK) return rc;
     argmax_final_kernel<<<dim3(1), dim3(1024), 0, s>>>((const unsigned long long *)workspace, gemv_blocks(vocab, rpw),
                                                        token, tokens, pos);
-    LLM_LAUNCH_CHECK("argmax_final_kernel");
-    return LLM_OK;
-}
-
-int llm_argmax_finish(const void *candidates, int n, int32_t *token, int32_t *tokens, int32_t *pos, llm_stream_t stream) {
-    LLM_REQUIRE(candidates && token && n > 0, "llm_argmax_finish: candidates/token/n");
-    LLM_REQUIRE((tokens == nullptr) == (pos == nullptr), "llm_argmax_finish: tokens and pos go together");
-    argmax_final_kernel<<<dim3(1), dim3(1024), 0, (hipStream_t)stream>>>((const unsigned long long *)candidates, n, token,
-                                                                         tokens, pos);
     LLM_LAUNCH_CHECK("argmax_final_kernel");
     return LLM_OK;
 }

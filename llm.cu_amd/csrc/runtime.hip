@@ -118,6 +118,14 @@ int llm_memcpy_d2d(void *dst, const void *src, size_t bytes, llm_stream_t s) {
     return copy(dst, src, bytes, hipMemcpyDeviceToDevice, s);
 }
 
+int llm_mem_info(size_t *free_bytes, size_t *total_bytes) {
+    size_t f = 0, t = 0;
+    LLM_HIP_CHECK(hipMemGetInfo(&f, &t));
+    if (free_bytes) *free_bytes = f;
+    if (total_bytes) *total_bytes = t;
+    return LLM_OK;
+}
+
 int llm_fill_zero(void *dst, size_t bytes, llm_stream_t stream) {
     LLM_REQUIRE((reinterpret_cast<uintptr_t>(dst) & 3u) == 0 && bytes % 4 == 0,
                 "llm_fill_zero needs 4-byte alignment and size");

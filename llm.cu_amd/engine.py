@@ -189,22 +189,18 @@ class Engine:
         lib().llama3_read_batch_logits(self.cache, b, out.ctypes.data)
         return out
 
-    def set_fused_decode(self, on):
-        """One launch per token (True, default where supported) or one launch per operation (False)."""
-        lib().llama3_set_fused_decode(self.cache, 1 if on else 0)
+    def set_handover(self, on, spin_limit=-1):
+        """Attention + output projection of a decode step in one launch (on) or one launch per operation."""
+        lib().llama3_set_handover(self.cache, 1 if on else 0, spin_limit)
 
-    @property
-    def fused_decode_active(self):
-        return bool(lib().llama3_fused_decode_active(self.cache))
+    def handover_stats(self):
+        """(waits that gave up, steps redone, hand-over launches in use)"""
+        t, r, a = C.c_long(0), C.c_long(0), C.c_int(0)
+        lib().llama3_handover_stats(self.cache, C.byref(t), C.byref(r), C.byref(a))
+        return t.value, r.value, bool(a.value)
 
-    def fused_vectors(self, which):
-        """Hand-over vectors of the last one-launch token: 0 qkv, 1 attention, 2 x after O, 3 FFN hidden, 4 layer output."""
-        c = self.cfg
-        qd = c.n_heads * c.head_dim
-        width = [qd + 2 * c.n_kv_heads * c.head_dim, qd, c.d_model, c.ffn_dim, c.d_model][which]
-        out = np.empty((c.n_layers, width), np.uint16)
-        lib().llama3_read_fused_vectors(self.cache, which, out.ctypes.data)
-        return out
+    def mark_handover_timeout(self):
+        lib().llama3_test_mark_handover_timeout(self.cache)
 
     def set_device_sampling(self, on):
         lib().llama3_set_device_sampling(self.cache, 1 if on else 0)

@@ -53,13 +53,12 @@ struct Engine {
     int32_t *d_token = nullptr;  // [0] last argmax, [1] waits of the fused attention + projection launch that gave up
     llm_half *ao_ring = nullptr; // one attention-output buffer per layer for llm_attn_decode_rope_oproj (null: not used)
     bool ao_long = false;        // the ring also serves llm_attn_decode_rope_long_oproj
-    // the whole decode token in one launch (llm_decode_fused), when the shapes and the device allow it
-    bool fused_ok = false, fused_on = false; // measured slower than one launch per operation: opt-in
-    llm_decode_desc fdesc = {};
-    llm_decode_layer *flayers = nullptr; // device array, rebuilt when the model changes
-    llm_half *fring[2] = {nullptr, nullptr};
-    void *fcand = nullptr;
-    int fset = 0; // buffer set of the next launch
+    // The launches that hand the attention output over inside the kernel are used while handover_on; a step in
+    // which a bounded wait gave up is redone with one launch per operation and the cache stays in that form.
+    bool handover_on = true;
+    int handover_spin_limit = -1; // < 0: the kernels' default
+    bool handover_test_mark = false; // tests: count one timeout into the next step as if a wait had given up
+    long handover_timeouts = 0, handover_recoveries = 0;
     void *ws_attn = nullptr, *ws_lm = nullptr;
     llm_half *trace_dev = nullptr;
     size_t trace_rows = 0;
@@ -83,8 +82,7 @@ struct Engine {
     long device_draws = 0, host_draws = 0;
     // one captured decode step per attention form: [0] single launch (up to 512 cached positions),
     // [1] span + merge launches (beyond)
-    // [2], [3]: the one-launch token working in buffer set 0 / 1
-    llm_graph_t graph[4] = {nullptr, nullptr, nullptr, nullptr};
+    llm_graph_t graph[2] = {nullptr, nullptr};
     bool long_attn = false; // form used by the next decode step that is issued
     // scratch of llama3_decode_batch (allocated by the first call on this cache as sequence 0)
     int batch_cap = 0;
@@ -146,31 +144,11 @@ void check_shapes(const Llama3 *m, const ModelConfig &c) {
 }
 
 void drop_graph(Engine *e) {
-    for (int f = 0; f < 4; ++f) {
+    for (int f = 0; f < 2; ++f) {
         if (!e->graph[f]) continue;
         llm_graph_destroy(e->graph[f]);
         e->graph[f] = nullptr;
     }
-}
-
-// Device table of per-layer pointers for llm_decode_fused; false when the q, k, v matrices of a layer
-// are not adjacent in memory (the one-launch token reads them as one matrix).
-bool build_fused_layers(Engine *e, const Llama3 *m) {
-    const ModelConfig &c = e->cfg;
-    const size_t qd = (size_t)c.n_heads * c.head_dim, kvd = (size_t)c.n_kv_heads * c.head_dim, d = c.d_model;
-    std::vector<llm_decode_layer> t(c.n_layers);
-    for (int l = 0; l < c.n_layers; ++l) {
-        const LayerW w = layer_w(m, l);
-        if (!(w.wk == w.wq + qd * d && w.wv == w.wk + kvd * d)) return false;
-        t[l] = {w.in_ln, w.wq, w.wo, w.post_ln, w.wg, w.wu, w.wd, e->kc + (size_t)l * e->kv_layer_elems,
-                e->vc + (size_t)l * e->kv_layer_elems};
-    }
-    if (!e->flayers) e->flayers = dmalloc<llm_decode_layer>(c.n_layers, "llm_malloc(layer table)");
-    llama3_check(llm_memcpy_h2d(e->flayers, t.data(), sizeof(llm_decode_layer) * t.size(), nullptr), "H2D layer table");
-    e->fdesc.embed_dev = m->embed_tokens->d_fp16_tensor;
-    e->fdesc.final_gain_dev = m->norm->d_fp16_tensor;
-    e->fdesc.lm_head_dev = m->lm_head->d_fp16_tensor;
-    return true;
 }
 
 // The captured decode graphs hold the weight pointers of the model they were captured with.  A call
@@ -183,10 +161,6 @@ void bind_model(Engine *e, const Llama3 *m) {
     drop_graph(e);
     e->model = m;
     e->model_slab = slab;
-    if (e->fring[0]) {
-        llama3_check(llm_stream_sync(e->stream), "stream sync"); // nothing in flight reads the old table
-        e->fused_ok = build_fused_layers(e, m);
-    }
 }
 
 // Issues one pass over T rows on the engine's stream.  With dev_pos the row
@@ -230,20 +204,20 @@ void issue_pass(Engine *e, const Llama3 *m, int T, int pos0, bool dev_pos, bool 
                 llama3_check(llm_norm_linear(e->x, w.in_ln, c.rms_eps, w.wv, e->qkv + qd + kvd, kvd, d, s),
                              "llm_norm_linear(v)");
             }
-            if (!e->long_attn && e->ao_ring) {
+            if (!e->long_attn && e->ao_ring && e->handover_on) {
                 // attention and output projection in one launch: the projection's weights stream while the
                 // attention runs.  Layer l hands over through ring buffer l and re-arms the next one.
                 llama3_check(llm_attn_decode_rope_oproj(e->qkv, kc, vc, e->ao_ring + (size_t)l * qd,
                                                         e->ao_ring + (size_t)((l + 1) % c.n_layers) * qd, p0, pd,
                                                         e->rope_table, Hq, Hkv, hd, c.max_pos, w.wo, e->x, e->x, d,
-                                                        e->d_token + 1, s),
+                                                        e->d_token + 1, e->handover_spin_limit, s),
                              "llm_attn_decode_rope_oproj");
-            } else if (e->long_attn && e->ao_ring && e->ao_long) {
+            } else if (e->long_attn && e->ao_ring && e->ao_long && e->handover_on) {
                 // long contexts: spans, then merge + output projection in one launch (same ring, same re-arming)
                 llama3_check(llm_attn_decode_rope_long_oproj(e->qkv, kc, vc, e->ao_ring + (size_t)l * qd,
                                                              e->ao_ring + (size_t)((l + 1) % c.n_layers) * qd, p0, pd,
                                                              e->rope_table, Hq, Hkv, hd, c.max_pos, e->ws_attn, w.wo, e->x,
-                                                             e->x, d, e->d_token + 1, s),
+                                                             e->x, d, e->d_token + 1, e->handover_spin_limit, s),
                              "llm_attn_decode_rope_long_oproj");
             } else {
                 llama3_check((e->long_attn ? llm_attn_decode_rope_long : llm_attn_decode_rope)(
@@ -294,9 +268,33 @@ void issue_pass(Engine *e, const Llama3 *m, int T, int pos0, bool dev_pos, bool 
 }
 
 // h_stage[3] mirrors d_token[1]: waits inside llm_attn_decode_rope_oproj that ran into their limit.  Any
-// such wait means a projection used an incomplete attention output: fail loudly.
-void check_handover(Engine *e) {
-    if (e->h_stage[3] != 0) llama3_fail("attention/projection hand-over timed out %d time(s)", e->h_stage[3]);
+// such wait means a projection used an incomplete attention output, so everything the step computed behind it
+// is invalid.  Returns false when the step is clean.  Otherwise the cache leaves the hand-over launches for
+// good (one launch per operation from here on: a device whose CUs are held by other work would run into the
+// limit again), the count is cleared, the buffers are armed again, the captured steps are dropped, and the
+// caller redoes the step: K and V rows of the position are simply written again.
+bool handover_gave_up(Engine *e) {
+    if (e->h_stage[3] == 0) return false;
+    if (!e->handover_on) llama3_fail("hand-over timeouts counted (%d) although no hand-over launch is in use", e->h_stage[3]);
+    fprintf(stderr, "[llama3] attention/projection hand-over gave up %d time(s) at position %d: redoing the step with one launch "
+                    "per operation (this cache keeps that form)\n", e->h_stage[3], e->pos);
+    e->handover_timeouts += e->h_stage[3];
+    ++e->handover_recoveries;
+    e->handover_on = false;
+    drop_graph(e);
+    llama3_check(llm_fill_zero(e->d_token + 1, sizeof(int32_t), e->stream), "zero timeout count");
+    llama3_check(llm_attn_oproj_buffer_init(e->ao_ring, e->cfg.n_layers * e->cfg.n_heads * e->cfg.head_dim, e->stream),
+                 "llm_attn_oproj_buffer_init");
+    e->h_stage[3] = 0;
+    return true;
+}
+
+// tests: the next step sees one counted timeout (the count only ever grows inside a step)
+void apply_test_mark(Engine *e) {
+    if (!e->handover_test_mark || !e->handover_on || !e->ao_ring) return;
+    e->handover_test_mark = false;
+    e->h_stage[4] = 1;
+    llama3_check(llm_memcpy_h2d(e->d_token + 1, &e->h_stage[4], sizeof(int32_t), e->stream), "H2D timeout mark");
 }
 
 // Brings the exp table and the selection buffers in line with the cache's sampler settings; false when
@@ -383,17 +381,22 @@ int run_pass(Engine *e, const Llama3 *m, const int *tokens, int n, llm_half *log
         }
         llama3_check(llm_memcpy_h2d(e->inject_dev, e->inject_host, sizeof(llm_half) * need, s), "H2D inject");
     }
-    e->long_attn = n == 1 && e->pos >= LONG_ATTN_FROM; // single rows go through the decode kernels
-    issue_pass(e, m, n, e->pos, false, trace, inject);
-    llama3_check(llm_memcpy_d2h(&e->h_stage[2], e->d_token, sizeof(int32_t) * 2, s), "D2H token");
-    if (trace)
-        llama3_check(llm_memcpy_d2h(e->trace_host, e->trace_dev, sizeof(llm_half) * (size_t)c.n_layers * n * c.d_model, s),
-                     "D2H trace");
-    if (logits_host)
-        llama3_check(llm_memcpy_d2h(logits_host, e->logits, sizeof(llm_half) * (size_t)c.vocab, s), "D2H logits");
-    if (e->select_pending) enqueue_selection(e, e->logits);
-    llama3_check(llm_stream_sync(s), "stream sync");
-    check_handover(e);
+    for (int attempt = 0;; ++attempt) {
+        if (attempt) // the first attempt's argmax advanced *d_pos
+            llama3_check(llm_memcpy_h2d(e->d_pos, &e->h_stage[1], sizeof(int32_t), s), "H2D position");
+        if (n == 1) apply_test_mark(e); // passes over several rows use no hand-over launch
+        e->long_attn = n == 1 && e->pos >= LONG_ATTN_FROM; // single rows go through the decode kernels
+        issue_pass(e, m, n, e->pos, false, trace, inject);
+        llama3_check(llm_memcpy_d2h(&e->h_stage[2], e->d_token, sizeof(int32_t) * 2, s), "D2H token");
+        if (trace)
+            llama3_check(llm_memcpy_d2h(e->trace_host, e->trace_dev, sizeof(llm_half) * (size_t)c.n_layers * n * c.d_model, s),
+                         "D2H trace");
+        if (logits_host)
+            llama3_check(llm_memcpy_d2h(logits_host, e->logits, sizeof(llm_half) * (size_t)c.vocab, s), "D2H logits");
+        if (e->select_pending) enqueue_selection(e, e->logits);
+        llama3_check(llm_stream_sync(s), "stream sync");
+        if (!handover_gave_up(e)) break;
+    }
     e->trace_host = nullptr;
     e->inject_host = nullptr;
     e->tokens.insert(e->tokens.end(), tokens, tokens + n);
@@ -415,36 +418,7 @@ void capture_decode_graph(Engine *e, const Llama3 *m, int form) {
 
 // pos: position of the token this step processes (known on the host although the kernels read it
 // from device memory), which selects the attention form
-// The whole token in one launch plus the argmax reduction, in buffer set `set`.
-void issue_fused_step(Engine *e, int set) {
-    llama3_check(llm_decode_fused(&e->fdesc, e->flayers, e->fring[set], e->fring[1 - set], 0, llm_decode_fused_phases(&e->fdesc),
-                                  e->d_token + 1, e->stream),
-                 "llm_decode_fused");
-    llama3_check(llm_argmax_finish(e->fcand, llm_decode_fused_candidates(&e->fdesc), e->d_token, e->d_tokens, e->d_pos,
-                                   e->stream),
-                 "llm_argmax_finish");
-}
-
-void capture_fused_graph(Engine *e, int set) {
-    llm_graph_t &g = e->graph[2 + set];
-    if (g) return;
-    llama3_check(llm_graph_capture_begin(e->stream), "graph capture begin");
-    issue_fused_step(e, set);
-    llama3_check(llm_graph_capture_end(e->stream, &g), "graph capture end");
-}
-
 void launch_decode_step(Engine *e, const Llama3 *m, int pos) {
-    if (pos < LONG_ATTN_FROM && e->fused_ok && e->fused_on) {
-        const int set = e->fset;
-        e->fset ^= 1; // consecutive tokens alternate the hand-over buffer sets
-        if (e->use_graph) {
-            capture_fused_graph(e, set);
-            llama3_check(llm_graph_launch(e->graph[2 + set], e->stream), "graph launch");
-        } else {
-            issue_fused_step(e, set);
-        }
-        return;
-    }
     const int form = pos >= LONG_ATTN_FROM ? 1 : 0;
     if (e->use_graph) {
         capture_decode_graph(e, m, form);
@@ -466,21 +440,25 @@ int step_one(Engine *e, const Llama3 *m, int token, llm_half *logits_host) {
     if (e->pos + 1 > c.max_pos) llama3_fail("sequence of %d tokens exceeds max_pos %d", e->pos + 1, c.max_pos);
     if (token < 0 || token >= c.vocab) llama3_fail("token id %d outside the vocabulary", token);
     llm_stream_t s = e->stream;
-    if (!e->dev_pos_valid || e->dev_next != token) {
-        e->h_stage[0] = token;
-        llama3_check(llm_memcpy_h2d(e->d_tokens + e->pos, &e->h_stage[0], sizeof(int32_t), s), "H2D token");
+    for (int attempt = 0;; ++attempt) {
+        if (attempt) e->dev_pos_valid = false; // a step that is redone starts from the host's view of the sequence
+        if (!e->dev_pos_valid || e->dev_next != token) {
+            e->h_stage[0] = token;
+            llama3_check(llm_memcpy_h2d(e->d_tokens + e->pos, &e->h_stage[0], sizeof(int32_t), s), "H2D token");
+        }
+        if (!e->dev_pos_valid) {
+            e->h_stage[1] = e->pos;
+            llama3_check(llm_memcpy_h2d(e->d_pos, &e->h_stage[1], sizeof(int32_t), s), "H2D position");
+        }
+        apply_test_mark(e);
+        launch_decode_step(e, m, e->pos);
+        llama3_check(llm_memcpy_d2h(&e->h_stage[2], e->d_token, sizeof(int32_t) * 2, s), "D2H token");
+        if (logits_host)
+            llama3_check(llm_memcpy_d2h(logits_host, e->logits, sizeof(llm_half) * (size_t)c.vocab, s), "D2H logits");
+        if (e->select_pending) enqueue_selection(e, e->logits);
+        llama3_check(llm_stream_sync(s), "stream sync");
+        if (!handover_gave_up(e)) break;
     }
-    if (!e->dev_pos_valid) {
-        e->h_stage[1] = e->pos;
-        llama3_check(llm_memcpy_h2d(e->d_pos, &e->h_stage[1], sizeof(int32_t), s), "H2D position");
-    }
-    launch_decode_step(e, m, e->pos);
-    llama3_check(llm_memcpy_d2h(&e->h_stage[2], e->d_token, sizeof(int32_t) * 2, s), "D2H token");
-    if (logits_host)
-        llama3_check(llm_memcpy_d2h(logits_host, e->logits, sizeof(llm_half) * (size_t)c.vocab, s), "D2H logits");
-    if (e->select_pending) enqueue_selection(e, e->logits);
-    llama3_check(llm_stream_sync(s), "stream sync");
-    check_handover(e);
     e->tokens.push_back(token);
     e->pos += 1;
     e->dev_pos_valid = true;
@@ -534,22 +512,6 @@ extern "C" CudaCache *init_cache_cfg(Llama3 *m, const ModelConfig *cfg) {
     }
     llama3_check(llm_fill_zero(e->d_tokens, sizeof(int32_t) * (R + 1), e->stream), "zero tokens");
     llama3_check(llm_fill_zero(e->d_pos, sizeof(int32_t), e->stream), "zero pos");
-    {
-        llm_decode_desc &f = e->fdesc;
-        f.n_layers = c.n_layers, f.d_model = d, f.n_heads = c.n_heads, f.n_kv_heads = c.n_kv_heads, f.head_dim = c.head_dim;
-        f.ffn_dim = c.ffn_dim, f.vocab = c.vocab, f.max_pos = c.max_pos, f.rms_eps = c.rms_eps;
-        f.rope_table_dev = e->rope_table, f.pos_dev = e->d_pos, f.tokens_dev = e->d_tokens, f.logits_dev = e->logits;
-        if (llm_decode_fused_supported(&f)) {
-            const size_t halves = llm_decode_fused_ring_halves(&f);
-            for (int i = 0; i < 2; ++i) {
-                e->fring[i] = dmalloc<llm_half>(halves, "llm_malloc(hand-over buffers)");
-                llama3_check(llm_attn_oproj_buffer_init(e->fring[i], (int)halves, e->stream), "arm hand-over buffers");
-            }
-            e->fcand = dmalloc<uint64_t>((size_t)llm_decode_fused_candidates(&f), "llm_malloc(argmax candidates)");
-            f.candidates_dev = e->fcand;
-            e->fused_ok = build_fused_layers(e, m);
-        }
-    }
     size_t wa = llm_attn_decode_workspace_bytes(c.n_heads, c.head_dim);
     wa = (wa + 3) / 4 * 4;
     llama3_check(llm_malloc(&e->ws_attn, wa), "llm_malloc(attention workspace)");
@@ -600,7 +562,7 @@ extern "C" void free_cache(CudaCache *C) {
         llm_stream_sync(e->stream);
         drop_graph(e);
         void *bufs[] = {e->x, e->xn, e->qkv, e->attn, e->ffn, e->logits, e->kc, e->vc, e->rope_table,
-                        e->d_tokens, e->d_pos, e->d_token, e->ao_ring, e->flayers, e->fring[0], e->fring[1], e->fcand, e->ws_attn, e->ws_lm, e->trace_dev, e->inject_dev,
+                        e->d_tokens, e->d_pos, e->d_token, e->ao_ring, e->ws_attn, e->ws_lm, e->trace_dev, e->inject_dev,
                         e->b_logits, e->b_ids, e->b_ws_attn, e->b_ws_argmax};
         for (void *b : bufs) llm_free(b);
         for (auto ev : e->ev) llm_event_destroy(ev);
@@ -666,27 +628,29 @@ extern "C" int llama3_generate(Llama3 *m, CudaCache *C, const int *prompt, int n
     // capture outside the timed decode region
     if (e->use_graph && n_decode > 1) {
         const int first_pos = start + n_prompt, last_pos = start + n_prompt + n_decode - 2;
-        if (first_pos < LONG_ATTN_FROM) {
-            if (e->fused_ok && e->fused_on) {
-                capture_fused_graph(e, 0);
-                capture_fused_graph(e, 1);
-            }
-            if (!(e->fused_ok && e->fused_on) || last_pos >= LONG_ATTN_FROM) capture_decode_graph(e, m, 0);
-        }
+        if (first_pos < LONG_ATTN_FROM) capture_decode_graph(e, m, 0);
         if (last_pos >= LONG_ATTN_FROM) capture_decode_graph(e, m, 1);
     }
-    llama3_check(llm_event_record(e->ev[2], s), "event record");
-    for (int i = 1; i < n_decode; ++i) launch_decode_step(e, m, start + n_prompt + i - 1);
-    llama3_check(llm_event_record(e->ev[3], s), "event record");
-    llama3_check(llm_stream_sync(s), "stream sync");
     out_tokens[0] = first;
-    if (n_decode > 1) {
+    for (int attempt = 0;; ++attempt) {
+        if (attempt) {
+            // a wait gave up somewhere in the run of steps: all of them again from the first decode position
+            // (d_tokens[first position] still holds the prompt pass's pick), now with one launch per operation
+            e->h_stage[1] = start + n_prompt;
+            llama3_check(llm_memcpy_h2d(e->d_pos, &e->h_stage[1], sizeof(int32_t), s), "H2D position");
+        }
+        if (n_decode > 1) apply_test_mark(e);
+        llama3_check(llm_event_record(e->ev[2], s), "event record");
+        for (int i = 1; i < n_decode; ++i) launch_decode_step(e, m, start + n_prompt + i - 1);
+        llama3_check(llm_event_record(e->ev[3], s), "event record");
+        llama3_check(llm_stream_sync(s), "stream sync");
+        if (n_decode <= 1) break;
         llama3_check(llm_memcpy_d2h(out_tokens + 1, e->d_tokens + start + n_prompt + 1,
                                     sizeof(int32_t) * (size_t)(n_decode - 1), s),
                      "D2H tokens");
         llama3_check(llm_memcpy_d2h(&e->h_stage[2], e->d_token, sizeof(int32_t) * 2, s), "D2H token");
         llama3_check(llm_stream_sync(s), "stream sync");
-        check_handover(e);
+        if (!handover_gave_up(e)) break;
     }
     // host mirror: the decode steps consumed out_tokens[0..n_decode-2]
     for (int i = 0; i + 1 < n_decode; ++i) e->tokens.push_back(out_tokens[i]);
@@ -810,27 +774,27 @@ extern "C" void llama3_read_logits(CudaCache *C, llm_half *logits) {
     llama3_check(llm_stream_sync(e->stream), "stream sync");
 }
 
-// Vectors that the last one-launch decode token handed over between its phases, for every layer:
-// which = 0 qkv, 1 attention output, 2 x after the O projection, 3 FFN hidden vector, 4 x after the down
-// projection (the layer's output).  out: [n_layers][width of that vector] fp16.
-extern "C" void llama3_read_fused_vectors(CudaCache *C, int which, llm_half *out) {
+// Hand-over launches of the decode step (attention and output projection in one launch): spin_limit < 0
+// restores the kernels' default bound of their wait, on != 0 puts a cache that left the form back into it.
+extern "C" void llama3_set_handover(CudaCache *C, int on, int spin_limit) {
     Engine *e = eng(C);
-    if (!e->fring[0] || which < 0 || which > 4) llama3_fail("llama3_read_fused_vectors: no one-launch token has run");
-    const ModelConfig &c = e->cfg;
-    const size_t qd = (size_t)c.n_heads * c.head_dim, qkv = qd + 2 * (size_t)c.n_kv_heads * c.head_dim, d = c.d_model;
-    const size_t F = c.ffn_dim, per_layer = qkv + qd + 2 * d + F;
-    const size_t off[5] = {0, qkv, qkv + qd, qkv + qd + d, qkv + qd + d + F}, width[5] = {qkv, qd, d, F, d};
-    const llm_half *set = e->fring[e->fset ^ 1]; // the set the last launch worked in
-    for (int l = 0; l < c.n_layers; ++l)
-        llama3_check(llm_memcpy_d2h(out + (size_t)l * width[which], set + per_layer * l + off[which],
-                                    sizeof(llm_half) * width[which], e->stream),
-                     "D2H hand-over vector");
-    llama3_check(llm_stream_sync(e->stream), "stream sync");
+    const bool want = on != 0;
+    if (want != e->handover_on || spin_limit != e->handover_spin_limit) {
+        llama3_check(llm_stream_sync(e->stream), "stream sync");
+        drop_graph(e);
+    }
+    e->handover_on = want;
+    e->handover_spin_limit = spin_limit;
 }
 
-extern "C" void llama3_set_fused_decode(CudaCache *C, int on) { eng(C)->fused_on = on != 0; }
+extern "C" void llama3_handover_stats(const CudaCache *C, long *timeouts, long *recoveries, int *active) {
+    const Engine *e = eng(C);
+    if (timeouts) *timeouts = e->handover_timeouts;
+    if (recoveries) *recoveries = e->handover_recoveries;
+    if (active) *active = (e->handover_on && e->ao_ring) ? 1 : 0;
+}
 
-extern "C" int llama3_fused_decode_active(const CudaCache *C) { return eng(C)->fused_ok && eng(C)->fused_on; }
+extern "C" void llama3_test_mark_handover_timeout(CudaCache *C) { eng(C)->handover_test_mark = true; }
 
 extern "C" void llama3_set_use_graph(CudaCache *C, int on) {
     Engine *e = eng(C);

@@ -202,8 +202,18 @@ def run_forced_parity(pkg, cfg, seed, n_prompt, n_decode):
         top = f16(lg_steps[same])
         out["free_divergence_gap"] = float(top[toks_o[same]] - top[out["tokens_gpu_free"][same]])
         out["free_divergence_logit_scale"] = float(np.abs(top).max())
+        # the engine's own logits at that step, on the same context (step by step up to the parting step):
+        # the two picks must be a near-tie by the engine's measured error at exactly those two logits
+        engine.reset()
+        t, _ = engine.prefill(prompt)
+        for i in range(same):
+            assert int(t) == toks_o[i]
+            t, _ = engine.decode(toks_o[i])
+        out["free_divergence_same_pick_stepwise"] = bool(int(t) == out["tokens_gpu_free"][same])
+        out["free_divergence_near_tie"] = bool(same_pick_or_near_tie(engine.logits(), lg_steps[same], int(t), toks_o[same]))
     else:
         out["free_divergence_gap"] = 0.0
+        out["free_divergence_near_tie"] = True
     o.close()
     engine.close()
     model.close()

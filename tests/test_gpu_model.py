@@ -175,48 +175,6 @@ def test_cache_follows_a_change_of_model(gpu):
     m2.close()
 
 
-@pytest.mark.parametrize("name,over,n_prompt,n_decode", [("tiny", dict(max_pos=128), 20, 40),
-                                                        ("tiny", dict(max_pos=1024), 490, 40),
-                                                        ("8b", dict(n_layers=2, max_pos=256), 33, 24),
-                                                        ("8b", dict(n_layers=3, max_pos=128), 7, 12)])
-def test_one_launch_token_equals_one_launch_per_operation(gpu, name, over, n_prompt, n_decode):
-    """llm_decode_fused (the whole decode token in one launch, vectors handed over inside the kernel) against
-    the per-operation launches: same greedy ids and, after every step, the same logits bit for bit; with and
-    without graph replay, through llama3_generate and through llama3_decode; the prompt of the second tiny
-    case ends at position 490, so its steps cross position 512 where the long-context kernels take over."""
-    cfg = gpu.engine.config(name, **over)
-    model = gpu.engine.Model.seeded(cfg, 61).to_device()
-    prompt = gpu.engine.seeded_tokens(61, n_prompt, cfg.vocab)
-    ref = gpu.engine.Engine(model, cfg, use_graph=False)
-    assert not ref.fused_decode_active   # opt-in: one launch per operation is the default (and the faster path)
-    want, _ = ref.generate(prompt, n_decode)
-    for use_graph in (True, False):
-        eng = gpu.engine.Engine(model, cfg, use_graph=use_graph)
-        eng.set_fused_decode(True)
-        assert eng.fused_decode_active
-        got, _ = eng.generate(prompt, n_decode)
-        assert list(got) == list(want), use_graph
-        assert np.array_equal(eng.logits(), ref.logits())
-        eng.reset()
-        got2, _ = eng.generate(prompt, n_decode)   # the hand-over buffers are back in their armed state
-        assert list(got2) == list(want)
-        eng.close()
-    # step by step, logits compared after every token
-    eng = gpu.engine.Engine(model, cfg, use_graph=True)
-    eng.set_fused_decode(True)
-    ref.reset()
-    t_e, _ = eng.prefill(prompt)
-    t_r, _ = ref.prefill(prompt)
-    for step in range(min(n_decode, 12)):
-        assert t_e == t_r
-        t_e, _ = eng.decode(t_e)
-        t_r, _ = ref.decode(t_r)
-        assert np.array_equal(eng.logits(), ref.logits()), step
-    eng.close()
-    ref.close()
-    model.close()
-
-
 def test_decode_across_the_long_context_attention_switch(gpu):
     """Greedy decoding from position 500 to 560 changes attention kernels at 512 cached positions (one
     launch before, span + merge launches after) and graphs with them: same ids with and without graphs,
@@ -498,24 +456,26 @@ def _check_forced(r):
     # where the free-running ids part from the oracle's (if they do), the oracle's own logits of the
     # two ids differ by less than the model tolerance of the logits
     assert r["free_divergence_gap"] <= 2 * tol * (1 + r.get("free_divergence_logit_scale", 0.0)), r["free_divergence_gap"]
+    # ... and by the engine's own logits at that step (same context) the two picks are the same id or a near-tie
+    assert r["free_divergence_near_tie"], r
+    assert r.get("free_divergence_same_pick_stepwise", True)
 
 
 def test_llama3_8b_full_depth_parity(gpu):
-    """All 32 layers of LLaMA3-8B on seeded weights (about 16 GB on each side), prompt of 32 ids, 32
+    """All 32 layers of LLaMA3-8B on seeded weights (about 16 GB on each side), prompt of 128 ids, 32
     greedy steps, against the ORC_REF16 oracle.  Random-init LLaMA at this depth amplifies one-ulp fp16
     rounding differences from layer to layer, so the comparison is made three ways (see
     helpers.run_forced_parity): layer by layer on identical inputs (asserted to 2e-2), free running
     (the engine's distance from unrounded arithmetic, ORC_FP32, asserted to be no more than 1.5x that of
     the reference's own rounding schedule), and on the greedy ids."""
-    cfg = gpu.engine.config("8b", max_pos=128)
+    cfg = gpu.engine.config("8b", max_pos=192)
     say("8B full depth: generating weights, oracle forward ...")
-    r = H.run_forced_parity(gpu, cfg, seed=2024, n_prompt=32, n_decode=32)
+    r = H.run_forced_parity(gpu, cfg, seed=2024, n_prompt=128, n_decode=32)
     say({k: (np.round(v, 4).tolist() if isinstance(v, list) and v and isinstance(v[0], float) else v)
          for k, v in r.items()})
     say("8B full depth: free-running greedy ids identical to the oracle's for the first",
         r["free_identical_prefix"], "of 32; oracle logit gap where they part:", r["free_divergence_gap"])
     _check_forced(r)
-    assert sum(a == b for a, b in zip(r["tokens_oracle"], r["tokens_gpu_forced"])) >= 30
 
 
 def test_tiny_forced_parity(gpu):

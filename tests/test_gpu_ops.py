@@ -316,6 +316,51 @@ def test_linear_mfma_8192_rows_sampled(gpu):
     assert np.array_equal(a[normal], b[normal])
 
 
+SAMPLED_ROWS = np.r_[0:32, 4080:4112, 8160:8192]   # first, middle and last row tiles of an 8192-row pass
+
+
+def test_o_projection_mfma_8192_rows_sampled(gpu):
+    """O projection of the 8192-token pass (K 4096 -> N 4096) with the residual added in place, as the engine
+    calls it; the oracle follows 96 of the rows."""
+    K, N, T = 4096, 4096, 8192
+    x, w = _proj_inputs(78, T, K, N)
+    res = H.bits(np.random.default_rng(79).standard_normal((T, N)))
+    got = gpu.ops.linear(x, w, residual=res, inplace=True)
+    want = orc.add(orc.linear(np.ascontiguousarray(x[SAMPLED_ROWS]), w), np.ascontiguousarray(res[SAMPLED_ROWS]))
+    e = H.mixed_err(got[SAMPLED_ROWS], want)
+    say("O 8192 err", e)
+    assert e <= TIGHT
+    assert np.array_equal(got, gpu.ops.linear(x, w, residual=res))   # in place == separate residual buffer
+
+
+def test_down_projection_mfma_8192_rows_sampled(gpu):
+    """Down projection of the 8192-token pass (K 14336 -> N 4096), residual in place."""
+    K, N, T = 14336, 4096, 8192
+    rng = np.random.default_rng(80)
+    x = H.bits(rng.standard_normal((T, K), dtype=np.float32))
+    w = H.bits(0.02 * rng.standard_normal((N, K), dtype=np.float32))
+    res = H.bits(rng.standard_normal((T, N), dtype=np.float32))
+    got = gpu.ops.linear(x, w, residual=res, inplace=True)
+    want = orc.add(orc.linear(np.ascontiguousarray(x[SAMPLED_ROWS]), w), np.ascontiguousarray(res[SAMPLED_ROWS]))
+    e = H.mixed_err(got[SAMPLED_ROWS], want)
+    say("down 8192 err", e)
+    assert e <= TIGHT
+
+
+def test_swiglu_mfma_8192_rows_sampled(gpu):
+    """Gate/up + SwiGLU of the 8192-token pass (K 4096 -> N 2 x 14336)."""
+    K, N, T = 4096, 14336, 8192
+    rng = np.random.default_rng(81)
+    x = H.bits(rng.standard_normal((T, K), dtype=np.float32))
+    wg = H.bits(0.02 * rng.standard_normal((N, K), dtype=np.float32))
+    wu = H.bits(0.02 * rng.standard_normal((N, K), dtype=np.float32))
+    got = gpu.ops.linear_swiglu(x, wg, wu)
+    want = orc.linear_swiglu(np.ascontiguousarray(x[SAMPLED_ROWS]), wg, wu)
+    e = H.mixed_err(got[SAMPLED_ROWS], want)
+    say("swiglu 8192 err", e)
+    assert e <= TOL
+
+
 # ---- LM head + argmax -----------------------------------------------------------------------------------------
 def test_lmhead_argmax_full_vocab(gpu):
     K, V = 4096, 128256
