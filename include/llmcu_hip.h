@@ -122,11 +122,19 @@ int llm_rope_kv_append(uint16_t *qkv_dev, uint16_t *k_cache_dev, uint16_t *v_cac
  * fp16(fp16(sum) + residual), the reference's add_norm applied to the stored
  * projection (inference.cu:377-390).  ldx/ldo/ldr are row strides in elements.
  * T == 1 runs the bandwidth-bound GEMV, 2 <= T <= 16 the skinny kernel, larger
- * T the MFMA GEMM.  K % 64 == 0 and N % 16 == 0 are required. */
+ * T the MFMA GEMM.  K % 64 == 0 and N % 16 == 0 are required.
+ * Device memory the call may take: passes of 17 to 1024 rows split k over several workgroups and keep fp32
+ * partial tiles in a 64 MiB buffer that belongs to the (device, stream) pair.  llm_init allocates the default
+ * stream's; any other stream gets its own at its first such launch (a hipMalloc inside llm_linear) and returns
+ * it in llm_stream_destroy -- a stream that was not created by llm_stream_create keeps its buffer until the
+ * process ends.  When the buffer cannot be had (no memory, or that first launch falls inside a graph capture)
+ * the launch runs unsplit, slower and with the same results up to summation order;
+ * llm_linear_unsplit_fallbacks() counts such launches since the library was loaded. */
 int llm_linear(const uint16_t *x_dev, int ldx, const uint16_t *w_dev, const uint16_t *residual_dev,
                int ldr, uint16_t *out_dev, int ldo, int T, int N, int K, llm_stream_t stream);
 /* Replaces kernel_standard_tiled_gemm_ffn_swiglu (src/inference/inference.cu:455-519):
  * out[t,n] = fp16(SiLU(sum_k x.wgate) * (sum_k x.wup)), neither sum rounded on its own. */
+long llm_linear_unsplit_fallbacks(void);
 int llm_linear_swiglu(const uint16_t *x_dev, int ldx, const uint16_t *wgate_dev,
                       const uint16_t *wup_dev, uint16_t *out_dev, int ldo, int T, int N, int K,
                       llm_stream_t stream);

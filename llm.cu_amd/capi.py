@@ -113,6 +113,7 @@ HIP_ABI = {
     "llm_rope": (_i, [_vp, _i, _i, _i, _i, _i, _vp, _vp, _i, _vp]),
     "llm_rope_kv_append": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _vp, _i, _vp]),
     "llm_linear": (_i, [_vp, _i, _vp, _vp, _i, _vp, _i, _i, _i, _i, _vp]),
+    "llm_linear_unsplit_fallbacks": (C.c_long, []),
     "llm_linear_swiglu": (_i, [_vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
     "llm_norm_linear": (_i, [_vp, _vp, C.c_double, _vp, _vp, _i, _i, _vp]),
     "llm_norm_linear_swiglu": (_i, [_vp, _vp, C.c_double, _vp, _vp, _vp, _i, _i, _vp]),

@@ -1001,9 +1001,12 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float *__restr
 // fp32 partial tiles of split-K launches: one 64 MB buffer per (device, stream), so that launches on
 // different streams never share partial sums.  llm_init allocates the default stream's buffer; any
 // other stream gets its own at its first split-K launch (these run at 17..1024 rows, never inside a
-// captured decode step) and gives it back in llm_stream_destroy.  Without a buffer (allocation failed)
-// the launch runs unsplit.
+// captured decode step) and gives it back in llm_stream_destroy.  Without a buffer (allocation failed, or the
+// stream's first split-K launch falls inside a graph capture, where nothing may be allocated) the launch runs
+// unsplit: same results up to summation order, fewer workgroups; g_unsplit_fallbacks counts those launches so
+// that a slow prompt pass can be traced to them (llm_linear_unsplit_fallbacks).
 static const size_t SPLITK_WS_BYTES = (size_t)64 << 20;
+static std::atomic<long> g_unsplit_fallbacks{0};
 struct SplitkWs {
     int device;
     hipStream_t stream;
@@ -1059,7 +1062,10 @@ static int gemm_dma_launch(const half_t *x, int ldx, const half_t *w, const half
     int rc = llm_ensure_max_smem((const void *)kern, smem, attr_done);
     if (rc != LLM_OK) return rc;
     float *ws = splits > 1 ? splitk_ws_for(s) : nullptr;
-    if (splits > 1 && !ws) splits = 1;
+    if (splits > 1 && !ws) {
+        splits = 1;
+        g_unsplit_fallbacks.fetch_add(1, std::memory_order_relaxed);
+    }
     if (splits > 1) {
         kern<<<dim3(tiles_m * tiles_n, splits), dim3(WGM * WGN * 64), smem, s>>>(x, ldx, w, w2, nullptr, 0, out, ldo, T, N, K,
                                                                                tiles_m, tiles_n, ws, K / splits);
@@ -1106,6 +1112,8 @@ static bool dma_ok(const half_t *out, int ldo, const half_t *res, int ldr, int T
 }
 
 extern "C" {
+
+long llm_linear_unsplit_fallbacks(void) { return g_unsplit_fallbacks.load(std::memory_order_relaxed); }
 
 int llm_linear(const uint16_t *x, int ldx, const uint16_t *w, const uint16_t *residual, int ldr, uint16_t *out,
                int ldo, int T, int N, int K, llm_stream_t stream) {

@@ -49,7 +49,7 @@ static ProbIndex *softmax_sorted(int vocab, float *tensor, const llm_half *half_
     float cumsum = 0.0f;
     for (int i = 0; i < vocab; ++i) {
         const float scaled = half_to_float(half_tensor[i]) / temperature;
-        tensor[i] = expf(scaled);
+        tensor[i] = expf(scaled); // the reference's exp(float) in a C++ translation unit is the float overload (inference.cu:1048)
         cumsum += tensor[i];
     }
     for (int i = 0; i < vocab; ++i) {

@@ -766,7 +766,11 @@ int orc_sample(const uint16_t *logits, int vocab, float temperature, int top_k, 
     const float rand_max = 2147483647.0f; /* (float)RAND_MAX */
     orc_prob *arr = (orc_prob *)malloc((size_t)vocab * sizeof(orc_prob));
     float *t = (float *)malloc((size_t)vocab * sizeof(float));
-    /* temperature_softmax, :1043-1072: no max subtraction, float running sum in index order */
+    /* temperature_softmax, :1043-1072: no max subtraction, float running sum in index order.  The
+     * reference writes exp(scaled_logit) with a float argument (:1048).  Its file is compiled as C++ (nvcc on a
+     * .cu file), where <cmath> overloads exp for float, so the call evaluates in single precision: expf here,
+     * which is C.  (Compiled as C the same text would promote to double and round the result to float: the two
+     * differ in the last bit for some arguments, and tests/test_sampler.py holds a case that tells them apart.) */
     float cumsum = 0.0f;
     for (int i = 0; i < vocab; ++i) {
         t[i] = expf(h2f(logits[i]) / temperature);

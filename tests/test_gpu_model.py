@@ -374,7 +374,7 @@ def test_errors_are_reported_not_swallowed(gpu):
     big = gpu.capi.DevBuf((1 << 16,), np.uint16)
     p = big.ptr
     for fn, extra in ((L.llm_attn_decode_rope_oproj, ()), (L.llm_attn_decode_rope_long_oproj, (p,))):
-        args = lambda out, nxt, pos, hq: (p, p, p, out, nxt, pos, None, p, hq, 2, 32, 64) + extra + (p, None, p, 64, p, None)
+        args = lambda out, nxt, pos, hq: (p, p, p, out, nxt, pos, None, p, hq, 2, 32, 64) + extra + (p, None, p, 64, p, -1, None)
         assert fn(*args(p, p, 3, 8)) == gpu.capi.LLM_ERR_INVALID and b"refill" in L.llm_last_error()
         assert fn(*args(p, p + 4096, 64, 8)) == gpu.capi.LLM_ERR_INVALID and b"position" in L.llm_last_error()
         assert fn(*args(p, p + 4096, 3, 6)) == gpu.capi.LLM_ERR_INVALID and b"not built" in L.llm_last_error()

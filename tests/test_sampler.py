@@ -160,6 +160,42 @@ def test_shipped_half_widening_all_patterns(pkg):
     lib.llama3_sampler_config(128256, 0.7, 50, 0.9)
 
 
+def test_exponentials_are_single_precision_as_in_a_cpp_translation_unit(pkg):
+    """inference.cu:1048 writes exp(float): compiled as C++ (nvcc on a .cu file) that is the float overload, not
+    a promotion to double.  Over every finite fp16 logit at temperature 0.7 the two readings differ in the last
+    bit for some patterns; the shipped temperature_softmax matches the single-precision reading bit for bit
+    (libm's expf, the running float sum in index order, then the division) and not the double one."""
+    lib = pkg.lib()
+    libm = C.CDLL("libm.so.6")
+    libm.expf.restype, libm.expf.argtypes = C.c_float, [C.c_float]
+    libm.exp.restype, libm.exp.argtypes = C.c_double, [C.c_double]
+    f = np.float32
+    allbits = np.arange(65536, dtype=np.uint16)
+    with np.errstate(invalid="ignore"):
+        vals = H.f16(allbits).astype(f)
+    keep = np.isfinite(vals) & (np.abs(vals) <= 20.0)
+    lg = np.ascontiguousarray(allbits[keep][::7])          # a few thousand patterns
+    scaled = (H.f16(lg).astype(f) / f(0.7)).astype(f)
+    single = np.array([libm.expf(float(x)) for x in scaled], dtype=f)
+    double = np.array([libm.exp(float(x)) for x in scaled]).astype(f)
+    differ = int(np.count_nonzero(single != double))
+    assert differ > 0                                        # otherwise this test could not tell the readings apart
+
+    def probabilities(e):
+        total = f(0)
+        for v in e:
+            total = f(total + v)
+        return (e / total).astype(f)
+
+    lib.llama3_sampler_config(lg.size, 0.7, 50, 0.9)
+    scratch = np.empty(lg.size, f)
+    arr = lib.temperature_softmax(scratch.ctypes.data, lg.ctypes.data, C.c_float(0.7))
+    C.CDLL("libc.so.6").free(C.c_void_p(arr))
+    lib.llama3_sampler_config(128256, 0.7, 50, 0.9)
+    assert np.array_equal(scratch, probabilities(single))
+    assert not np.array_equal(scratch, probabilities(double))
+
+
 def test_fast_head_selection_equals_the_full_sort_path(pkg):
     """sample_next_token() selects only the top-k head; sample_next_token_reference() is the reference's
     call sequence with the full qsort.  fp16 logits at vocabulary size tie constantly, so the order among

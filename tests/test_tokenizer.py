@@ -139,3 +139,67 @@ def test_failures_print_and_exit_like_the_reference(tmp_path):
     # the reference's own entry point looks for model_weights/modified_tokenizer.json
     p = _child("lib.load_tokenizer()")
     assert p.returncode == 1 and "Could not determine file size" in p.stdout
+
+
+class _Node(C.Structure):
+    pass
+
+
+_Node._fields_ = [("_max_childs", C.c_int), ("child_len", C.c_int), ("child_char", C.POINTER(C.c_ubyte)),
+                  ("child_node", C.POINTER(C.POINTER(_Node))), ("token", C.c_int)]
+
+
+def _walk(node, prefix, out):
+    """every (string, id) a trie holds; checks the ordering invariant and the capacity on the way"""
+    n = node.contents
+    assert 0 <= n.child_len <= n._max_childs
+    bytes_ = [n.child_char[i] for i in range(n.child_len)]
+    assert bytes_ == sorted(set(bytes_)), bytes_          # ascending unsigned bytes, no duplicates
+    if n.token != -1:
+        out[bytes(prefix)] = n.token
+    for i in range(n.child_len):
+        _walk(n.child_node[i], prefix + [bytes_[i]], out)
+
+
+def test_trie_built_at_once_and_string_by_string_hold_the_same_vocabulary(pkg, tmp_path):
+    """The loader lays the trie down from the sorted vocabulary in one pass; the exported _build_trie splices
+    one string at a time into place.  Both keep a node's children sorted by unsigned byte (what _find_child's
+    binary search needs) and both hold exactly the oracle's vocabulary, whatever the insertion order; a trie
+    made by hand tokenizes like the loaded one."""
+    lib = _lib(pkg)
+    path = str(tmp_path / "tokenizer.json")
+    _write_tokenizer(path)
+    enc, _ = tok_orc.load_vocab(path)
+    tk = lib.load_tokenizer_from(path.encode(), DECODE_SIZE)
+
+    class Tok(C.Structure):
+        _fields_ = [("root", C.POINTER(_Node)), ("decode", C.c_void_p)]
+
+    loaded = {}
+    _walk(C.cast(tk, C.POINTER(Tok)).contents.root, [], loaded)
+    assert loaded == enc
+    lib.init_trienode.restype = C.POINTER(_Node)
+    lib._build_trie.argtypes = [C.POINTER(_Node), C.c_char_p, C.c_int]
+    lib._find_child.argtypes = [C.POINTER(_Node), C.c_char, C.POINTER(C.POINTER(_Node))]
+    rng = np.random.default_rng(4)
+    items = list(enc.items())
+    for trial in range(3):
+        order = rng.permutation(len(items))
+        root = lib.init_trienode()
+        lib._build_trie(root, b"the", 12345)              # replaced below: the later definition of a string stays
+        for j in order:
+            lib._build_trie(root, items[j][0], items[j][1])
+        built = {}
+        _walk(root, [], built)
+        assert built == enc
+        hit = C.POINTER(_Node)()
+        assert lib._find_child(root, b"t", C.byref(hit)) >= 0 and lib._find_child(root, b"\x01", C.byref(hit)) == -1
+        assert lib._find_child(root, "日".encode()[:1], C.byref(hit)) >= 0     # a byte above 0x7f
+        hand = Tok(root, None)
+        libc = C.CDLL("libc.so.6")
+        for text in (b"there and here", "日本語 ée".encode(), b"<|eot_id|>the abcd"):
+            a, b = lib.tokenize(C.byref(hand), text), lib.tokenize(tk, text)
+            assert [a[i] for i in range(a[0])] == [b[i] for i in range(b[0])]
+            libc.free(a)
+            libc.free(b)
+    lib.free_tokenizer(tk, DECODE_SIZE)
