@@ -216,7 +216,7 @@ __global__ __launch_bounds__(AD_THREADS) void attn_oproj_kernel(const int32_t *p
         if (pos > AD_LS - 1) pos = AD_LS - 1; // this form serves one span; the host picks it below AD_LS only
         if (pos < 0) pos = 0;
         const int kvh = wg % a.n_kv_heads, y = wg / a.n_kv_heads;
-        attn_decode_body<HD, G, true, HD / DSN, AD_LS, false, true>(a, sc, qs, knew, vnew, s_m, s_l, &s_last, pos, 1, 0,
+        attn_decode_body<HD, G, true, HD / DSN, AD_LS, true>(a, sc, qs, knew, vnew, s_m, s_l, &s_last, pos, 1, 0,
                                                                     y * (HD / DSN), y == 0, kvh);
         // off the critical path: the next launch's buffer back to "empty" (visible at the end of this kernel)
         uint32_t *nx = reinterpret_cast<uint32_t *>(o.next);
@@ -288,50 +288,41 @@ static int dispatch_decode(AdArgs a, int n_heads, int head_dim, void *ws, hipStr
 }
 
 // ---------------------------------------------------------------------------
-// Long contexts: two launches.  attn_span_kernel gives every (KV head, 256-position span) its own
-// workgroup and leaves (max, sum, unnormalised P.V) per span; attn_merge_kernel, one workgroup per
-// query head, combines them.  No fence, counter or last-workgroup tail: beyond a few spans that tail
+// Long contexts: two launches.  attn_span_kernel gives every (KV head, span of positions) its own
+// workgroup (attn_span_wave: eight wavefronts of 32 positions, each on its own until the combine; two
+// workgroups fit a CU) and leaves (max, sum, unnormalised P.V) per span; attn_merge_kernel, one workgroup
+// per query head, combines them.  No fence, counter or last-workgroup tail: beyond a few spans that tail
 // costs more than the second launch.
 // ---------------------------------------------------------------------------
-#define AD_LONG_LS 256      // shortest span of the long form (ad_long_span_len)
-#define AD_LONG_LS_MAX 512  // longest
 #define AD_MERGE_THREADS 512
 
 // (arguments as leading scalars, like attn_oproj_kernel: kvh_maxpos = n_kv_heads | max_pos << 8,
 // splits_target = splits | span_target << 16)
-template <int HD, int G, bool FUSED>
-__global__ __launch_bounds__(AD_THREADS) void attn_span_kernel(const int32_t *pos_dev, const half_t *q, half_t *kc,
-                                                               half_t *vc, const float *table, int pos_host,
-                                                               int kvh_maxpos, int splits_target, float *ws_acc,
-                                                               float *ws_ml) {
+template <int HD, int G>
+__global__ __launch_bounds__(AD_SPAN_THREADS, 4) void attn_span_kernel(const int32_t *pos_dev, const half_t *q, half_t *kc,
+                                                                  half_t *vc, const float *table, int pos_host,
+                                                                  int kvh_maxpos, int splits_target, float *ws_acc,
+                                                                  float *ws_ml) {
     AdArgs a = {};
     a.q = q;
     a.kc = kc;
     a.vc = vc;
     a.table = table;
-    a.pos_host = pos_host;
-    a.pos_dev = pos_dev;
     a.n_kv_heads = kvh_maxpos & 0xff;
     a.max_pos = (int)((unsigned)kvh_maxpos >> 8);
     a.splits = splits_target & 0xffff;
     a.span_target = (int)((unsigned)splits_target >> 16);
     a.ws_acc = ws_acc;
     a.ws_ml = ws_ml;
-    __shared__ float sc[G * AD_LONG_LS];
-    __shared__ __attribute__((aligned(16))) half_t qs[G * HD];
-    __shared__ __attribute__((aligned(16))) half_t knew[HD];
-    __shared__ __attribute__((aligned(16))) half_t vnew[HD];
-    __shared__ float s_m[G], s_l[G];
-    __shared__ int s_last;
-    int pos = a.pos_host + (a.pos_dev ? *a.pos_dev : 0);
+    int pos = pos_host + (pos_dev ? *pos_dev : 0);
     if (pos > a.max_pos - 1) pos = a.max_pos - 1;
     if (pos < 0) pos = 0;
-    const int span_len = ad_long_span_len(pos + 1, a.span_target);
-    const int n_active = ad_long_spans(pos + 1, a.span_target);
+    const int span = ad_long_span(pos + 1, a.span_target);
+    const int n_active = (pos + span) / span;
     const int y = blockIdx.y;
     if (y >= n_active) return;
-    attn_decode_body<HD, G, FUSED, HD, AD_LONG_LS_MAX, true>(a, sc, qs, knew, vnew, s_m, s_l, &s_last, pos, n_active, y, 0,
-                                                             y == n_active - 1, -1, span_len);
+    if (y == n_active - 1) attn_span_wave<HD, G, true>(a, pos, y, blockIdx.x, span);
+    else attn_span_wave<HD, G, false>(a, pos, y, blockIdx.x, span);
 }
 
 // AGENT_OUT: the head's result leaves as 8-byte device-scope stores with the "not written yet" pattern avoided,
@@ -418,29 +409,24 @@ __global__ __launch_bounds__(AD_MERGE_THREADS) void attn_merge_kernel(const AdAr
     attn_merge_body<HD, G>(a, blockIdx.x);
 }
 
-// Long form on the host: the span target of this device (a.span_target) and the second grid dimension of the span
-// kernel (the spans in use when the position is known here, else the most that any position below max_pos needs).
+// Long form on the host: the span target of this device (a.span_target), the span count of the workspace layout
+// (a.splits: never fewer than any position below max_pos uses) and the second grid dimension of the span kernel
+// (the spans in use when the position is known here, else that same upper bound).
 static int ad_long_setup(AdArgs &a, int *gy) {
     int cus = 0;
     int rc = llm_cu_count_cached(&cus);
     if (rc != LLM_OK) return rc;
-    a.span_target = cus / a.n_kv_heads > 0 ? cus / a.n_kv_heads : 1;
-    const int splits = (a.max_pos + AD_LONG_LS - 1) / AD_LONG_LS; // spans of the workspace layout: never fewer than in use
-    LLM_REQUIRE(splits <= AD_MAX_SPLITS, "decode attention: max_pos=%d exceeds %d", a.max_pos, AD_MAX_SPLITS * AD_LONG_LS);
+    int target = cus / a.n_kv_heads;
+    a.span_target = target < 1 ? 1 : target > 64 ? 64 : target;
+    const int splits = ad_long_max_spans(a.max_pos, a.span_target);
+    LLM_REQUIRE(splits <= AD_MAX_SPLITS, "decode attention: max_pos=%d exceeds %d", a.max_pos, AD_MAX_SPLITS * AD_SPAN);
     a.splits = splits;
-    LLM_REQUIRE(a.n_kv_heads < 256 && a.max_pos < (1 << 23) && a.span_target < (1 << 15), "decode attention: %d kv heads, max_pos %d",
-                a.n_kv_heads, a.max_pos);
-    if (a.pos_dev) {
-        const int knee = a.span_target * AD_LONG_LS < a.max_pos ? a.span_target * AD_LONG_LS : a.max_pos;
-        const int m1 = ad_long_spans(knee, a.span_target), m2 = ad_long_spans(a.max_pos, a.span_target);
-        *gy = m1 > m2 ? m1 : m2;
-    } else {
-        *gy = ad_long_spans(a.pos_host + 1, a.span_target);
-    }
+    LLM_REQUIRE(a.n_kv_heads < 256 && a.max_pos < (1 << 23), "decode attention: %d kv heads, max_pos %d", a.n_kv_heads, a.max_pos);
+    *gy = a.pos_dev ? splits : ad_long_spans(a.pos_host + 1, a.span_target);
     return LLM_OK;
 }
 
-template <int HD, int G, bool FUSED>
+template <int HD, int G>
 static int launch_decode_long(AdArgs a, void *ws, hipStream_t s) {
     const int Hq = a.n_kv_heads * G;
     a.ws_acc = (float *)ws;
@@ -449,7 +435,7 @@ static int launch_decode_long(AdArgs a, void *ws, hipStream_t s) {
     int gy = 0;
     int rc = ad_long_setup(a, &gy);
     if (rc != LLM_OK) return rc;
-    attn_span_kernel<HD, G, FUSED><<<dim3(a.n_kv_heads, gy), dim3(AD_THREADS), 0, s>>>(
+    attn_span_kernel<HD, G><<<dim3(a.n_kv_heads, gy), dim3(AD_SPAN_THREADS), 0, s>>>(
         a.pos_dev, a.q, a.kc, a.vc, a.table, a.pos_host, a.n_kv_heads | (a.max_pos << 8), a.splits | (a.span_target << 16), a.ws_acc,
         a.ws_ml);
     LLM_LAUNCH_CHECK("attn_span_kernel");
@@ -520,7 +506,7 @@ static int launch_long_oproj(AdArgs a, AoArgs o, void *ws, hipStream_t s) {
     int gy = 0;
     rc = ad_long_setup(a, &gy);
     if (rc != LLM_OK) return rc;
-    attn_span_kernel<HD, G, true><<<dim3(a.n_kv_heads, gy), dim3(AD_THREADS), 0, s>>>(
+    attn_span_kernel<HD, G><<<dim3(a.n_kv_heads, gy), dim3(AD_SPAN_THREADS), 0, s>>>(
         a.pos_dev, a.q, a.kc, a.vc, a.table, a.pos_host, a.n_kv_heads | (a.max_pos << 8), a.splits | (a.span_target << 16), a.ws_acc,
         a.ws_ml);
     LLM_LAUNCH_CHECK("attn_span_kernel");
@@ -578,20 +564,14 @@ __global__ __launch_bounds__(AD_THREADS) void attn_decode_batch_kernel(const AdA
 }
 
 template <int HD, int G>
-__global__ __launch_bounds__(AD_THREADS) void attn_span_batch_kernel(const AdArgs common, const AdBatch b) {
-    __shared__ float sc[G * AD_LONG_LS];
-    __shared__ __attribute__((aligned(16))) half_t qs[G * HD];
-    __shared__ __attribute__((aligned(16))) half_t knew[HD];
-    __shared__ __attribute__((aligned(16))) half_t vnew[HD];
-    __shared__ float s_m[G], s_l[G];
-    __shared__ int s_last;
+__global__ __launch_bounds__(AD_SPAN_THREADS, 4) void attn_span_batch_kernel(const AdArgs common, const AdBatch b) {
     const AdArgs a = ad_for_sequence(common, b, blockIdx.z);
-    const int span_len = ad_long_span_len(a.pos_host + 1, a.span_target);
-    const int n_active = ad_long_spans(a.pos_host + 1, a.span_target);
+    const int span = ad_long_span(a.pos_host + 1, a.span_target);
+    const int n_active = (a.pos_host + span) / span;
     const int y = blockIdx.y;
     if (y >= n_active) return;
-    attn_decode_body<HD, G, true, HD, AD_LONG_LS_MAX, true>(a, sc, qs, knew, vnew, s_m, s_l, &s_last, a.pos_host, n_active,
-                                                            y, 0, y == n_active - 1, -1, span_len);
+    if (y == n_active - 1) attn_span_wave<HD, G, true>(a, a.pos_host, y, blockIdx.x, span);
+    else attn_span_wave<HD, G, false>(a, a.pos_host, y, blockIdx.x, span);
 }
 
 template <int HD, int G>
@@ -623,18 +603,17 @@ static int launch_decode_batch(AdArgs a, const AdBatch &b, int B, void *ws, hipS
         const int n = ad_long_spans(b.pos[z] + 1, a.span_target);
         gy = n > gy ? n : gy;
     }
-    attn_span_batch_kernel<HD, G><<<dim3(a.n_kv_heads, gy, B), dim3(AD_THREADS), 0, s>>>(a, b);
+    attn_span_batch_kernel<HD, G><<<dim3(a.n_kv_heads, gy, B), dim3(AD_SPAN_THREADS), 0, s>>>(a, b);
     LLM_LAUNCH_CHECK("attn_span_batch_kernel");
     attn_merge_batch_kernel<HD, G><<<dim3(Hq, B), dim3(AD_MERGE_THREADS), 0, s>>>(a, b);
     LLM_LAUNCH_CHECK("attn_merge_batch_kernel");
     return LLM_OK;
 }
 
-template <bool FUSED>
 static int dispatch_decode_long(AdArgs a, int n_heads, int head_dim, void *ws, hipStream_t s) {
     const int G = n_heads / a.n_kv_heads;
 #define AD_CASE(HD_, G_) \
-    if (head_dim == HD_ && G == G_) return launch_decode_long<HD_, G_, FUSED>(a, ws, s);
+    if (head_dim == HD_ && G == G_) return launch_decode_long<HD_, G_>(a, ws, s);
     AD_CASE(128, 4)
     AD_CASE(128, 8)
     AD_CASE(128, 1)
@@ -874,7 +853,7 @@ int llm_attn_decode_rope_long(const uint16_t *qkv, uint16_t *kc, uint16_t *vc, u
     a.pos_dev = pos_dev;
     a.n_kv_heads = n_kv_heads;
     a.max_pos = max_pos;
-    return dispatch_decode_long<true>(a, n_heads, head_dim, workspace, (hipStream_t)stream);
+    return dispatch_decode_long(a, n_heads, head_dim, workspace, (hipStream_t)stream);
 }
 
 // 1 when llm_attn_decode_rope_long_oproj covers these shapes on the current device, else 0.
