@@ -94,10 +94,17 @@ struct AoArgs {
     int spin_limit;    // polling rounds before a wait gives up
 };
 
-// The projection role of a launch whose first n_first workgroups produce the projection's input vector (a.out,
-// handed over as described above): all weight rows of the workgroup are requested at once, then the vector is
-// polled for, staged in xs (K halves of LDS) and reduced against.
-__device__ __forceinline__ void ao_projection_part(const AdArgs &a, const AoArgs &o, half_t *xs, const int n_attn) {
+// The projection role of a launch some of whose workgroups produce the projection's input vector (a.out, handed
+// over as described above): all weight rows of the workgroup are requested at once (ao_projection_loads), then the
+// vector is polled for, staged in LDS and reduced against (ao_projection_finish).  n_attn: workgroups in front
+// that take no rows.
+struct AoRows {
+    half8_t wreg[AO_ROWS][AO_KSTEPS];
+    half_t resv[AO_ROWS];
+};
+
+// first half: the weight rows (and residual values) of this workgroup, all asked for at once
+__device__ __forceinline__ void ao_projection_loads(const AoArgs &o, const int n_attn, const int head_start, AoRows &R) {
     const int wg = blockIdx.x, tid = threadIdx.x;
     const int wave = tid / 64, lane = tid % 64;
     const int K = o.K, N = o.N;
@@ -107,11 +114,10 @@ __device__ __forceinline__ void ao_projection_part(const AdArgs &a, const AoArgs
     // and 16 to the others.
     const int wslot = (wg - n_attn) + o.n_owg * wave;
     const int wtotal = o.n_owg * AO_WAVES;
-    half8_t wreg[AO_ROWS][AO_KSTEPS];
-    half_t resv[AO_ROWS];
-    // a head start of a little under a microsecond for the attention's own loads (measured per launch: 12.2 -> 11.4 us
-    // with the first version of the attention; against the current one three pauses beat 0-2 and 4-8)
-    for (int dl = 0; dl < 3; ++dl) __builtin_amdgcn_s_sleep(8);
+    // (attention + projection launch: a head start of a little under a microsecond for the attention's own loads,
+    // measured per launch: 12.2 -> 11.4 us with the first version of the attention; against the current one three
+    // pauses beat 0-2 and 4-8)
+    for (int dl = 0; dl < head_start; ++dl) __builtin_amdgcn_s_sleep(8);
 #pragma unroll
     for (int r = 0; r < AO_ROWS; ++r) {
         int row = wslot + wtotal * r;
@@ -120,10 +126,20 @@ __device__ __forceinline__ void ao_projection_part(const AdArgs &a, const AoArgs
 #pragma unroll
         for (int j = 0; j < AO_KSTEPS; ++j) {
             const int k = lane * 8 + 512 * j;
-            wreg[r][j] = (live && k < K) ? load8_nt(o.w + (size_t)row * K + k) : half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+            R.wreg[r][j] = (live && k < K) ? load8_nt(o.w + (size_t)row * K + k) : half8_t{0, 0, 0, 0, 0, 0, 0, 0};
         }
-        resv[r] = (live && o.res) ? o.res[row] : (half_t)0.f;
+        R.resv[r] = (live && o.res) ? o.res[row] : (half_t)0.f;
     }
+}
+
+// second half: wait for the input vector (a.out, handed over as described above), stage it in xs (K halves of
+// LDS), reduce the rows against it and store
+__device__ __forceinline__ void ao_projection_finish(const AdArgs &a, const AoArgs &o, half_t *xs, const int n_attn, const AoRows &R) {
+    const int wg = blockIdx.x, tid = threadIdx.x;
+    const int wave = tid / 64, lane = tid % 64;
+    const int K = o.K, N = o.N;
+    const int wslot = (wg - n_attn) + o.n_owg * wave;
+    const int wtotal = o.n_owg * AO_WAVES;
     // ---- the attention output, as soon as it is there ------------------------------------
     {
         const uint32_t *src = reinterpret_cast<const uint32_t *>(a.out);
@@ -165,7 +181,7 @@ __device__ __forceinline__ void ao_projection_part(const AdArgs &a, const AoArgs
         if (k < K) {
             const half8_t x = load8(xs + k);
 #pragma unroll
-            for (int r = 0; r < AO_ROWS; ++r) acc[r] = dot8(wreg[r][j], x, acc[r]);
+            for (int r = 0; r < AO_ROWS; ++r) acc[r] = dot8(R.wreg[r][j], x, acc[r]);
         }
     }
 #pragma unroll
@@ -175,7 +191,7 @@ __device__ __forceinline__ void ao_projection_part(const AdArgs &a, const AoArgs
         const int row = wslot + wtotal * r;
         if (lane == 0 && r < o.rows && row < N) {
             half_t h = (half_t)acc[r];
-            if (o.res) h = (half_t)((float)h + (float)resv[r]); // the reference's add_norm on the stored projection
+            if (o.res) h = (half_t)((float)h + (float)R.resv[r]); // the reference's add_norm on the stored projection
             o.out[row] = h;
         }
     }
@@ -223,7 +239,9 @@ __global__ __launch_bounds__(AD_THREADS) void attn_oproj_kernel(const int32_t *p
         for (int c = wg * AD_THREADS + tid; c < o.K / 2; c += n_attn * AD_THREADS) nx[c] = AO_EMPTY | (AO_EMPTY << 16);
         return;
     }
-    ao_projection_part(a, o, reinterpret_cast<half_t *>(sc), n_attn); // K halves: K * 2 <= sizeof(sc), checked by the host
+    AoRows R;
+    ao_projection_loads(o, n_attn, 3, R);
+    ao_projection_finish(a, o, reinterpret_cast<half_t *>(sc), n_attn, R); // K halves: K * 2 <= sizeof(sc), checked by the host
 }
 
 template <int HD, int G>
@@ -472,13 +490,17 @@ __global__ __launch_bounds__(AD_THREADS) void merge_oproj_kernel(const int32_t *
     __shared__ __attribute__((aligned(16))) half_t xs[AO_KSTEPS * 512];
     const int n_first = a.n_kv_heads * G;
     const int wg = blockIdx.x, tid = threadIdx.x;
+    // (The merging workgroups take no projection rows: a wavefront's loads come back in order, so the reads of the
+    // spans' partial results would stand behind its weight rows -- measured 1.7 us per launch slower.)
     if (wg < n_first) {
         attn_merge_body<HD, G, true>(a, wg);
         uint32_t *nx = reinterpret_cast<uint32_t *>(o.next);
         for (int c = wg * AD_THREADS + tid; c < o.K / 2; c += n_first * AD_THREADS) nx[c] = AO_EMPTY | (AO_EMPTY << 16);
         return;
     }
-    ao_projection_part(a, o, xs, n_first);
+    AoRows R;
+    ao_projection_loads(o, n_first, 0, R);
+    ao_projection_finish(a, o, xs, n_first, R);
 }
 
 // projection workgroups and rows per wavefront behind n_first producer workgroups; false when they do not fit
