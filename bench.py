@@ -186,7 +186,7 @@ def main():
         batched = {}
         bcfg = eng_mod.config("8b", max_pos=512)
         for B in (4, 16):
-            engines = [eng_mod.Engine(model, bcfg, use_graph=False) for _ in range(B)]
+            engines = [eng_mod.Engine(model, bcfg) for _ in range(B)]
             cur = []
             for b, e in enumerate(engines):
                 t, _ = e.prefill(eng_mod.seeded_tokens(a.seed + 10 + b, a.prompt, bcfg.vocab))

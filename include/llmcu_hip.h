@@ -251,6 +251,20 @@ int llm_attn_decode_rope_batch(const uint16_t *qkv_dev, int ldq, uint16_t *const
                                const int *positions, int batch, uint16_t *out_dev, int ldo, const float *table_dev,
                                int n_heads, int n_kv_heads, int head_dim, int max_pos, void *workspace_dev,
                                llm_stream_t stream);
+/* The same with the caches and positions of the sequences read from device memory when the kernels run, so that
+ * the launch can be captured once and replayed while the sequences advance: desc_dev points to an llm_batch_desc in
+ * device memory (the caller rewrites it between replays, in stream order); cache_offset is added, in elements, to
+ * every cache pointer (a layer's part of caches that hold all layers).  long_form: 0 when every position is below
+ * 512 (one launch), 1 otherwise (span + merge launches, grids sized for any position below max_pos); positions are
+ * clamped to what the chosen form serves. */
+#define LLM_MAX_BATCH 16
+typedef struct {
+    uint16_t *k_cache[LLM_MAX_BATCH], *v_cache[LLM_MAX_BATCH];
+    int32_t pos[LLM_MAX_BATCH];
+} llm_batch_desc;
+int llm_attn_decode_rope_batch_dev(const uint16_t *qkv_dev, int ldq, const llm_batch_desc *desc_dev, size_t cache_offset,
+                                   int batch, int long_form, uint16_t *out_dev, int ldo, const float *table_dev, int n_heads,
+                                   int n_kv_heads, int head_dim, int max_pos, void *workspace_dev, llm_stream_t stream);
 /* Same attention for T query rows at positions pos0..pos0+T-1 (prompt pass),
  * streaming softmax on MFMA tiles; never materialises [H,T,T].
  * q: [T, ldq] with head h at columns h*hd; out: [T, ldo].  Cache rows beyond

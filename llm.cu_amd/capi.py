@@ -120,6 +120,7 @@ HIP_ABI = {
     "llm_embed_norm_linear": (_i, [_vp, _vp, _vp, _i, _vp, _vp, C.c_double, _vp, _vp, _i, _i, _vp]),
     "llm_attn_decode_rope": (_i, [_vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _vp, _vp]),
     "llm_attn_decode_rope_batch": (_i, [_vp, _i, _vp, _vp, _vp, _i, _vp, _i, _vp, _i, _i, _i, _i, _vp, _vp]),
+    "llm_attn_decode_rope_batch_dev": (_i, [_vp, _i, _vp, _sz, _i, _i, _vp, _i, _vp, _i, _i, _i, _i, _vp, _vp]),
     "llm_attn_oproj_supported": (_i, [_i, _i, _i, _i]),
     "llm_attn_oproj_buffer_init": (_i, [_vp, _i, _vp]),
     "llm_attn_decode_rope_oproj": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _vp, _vp, _vp, _i, _vp, _i, _vp]),

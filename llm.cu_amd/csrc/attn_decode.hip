@@ -555,13 +555,33 @@ struct AdBatch {
     size_t ws_floats;  // workspace floats per sequence (long form)
 };
 
-__device__ __forceinline__ AdArgs ad_for_sequence(const AdArgs &common, const AdBatch &b, int z) {
-    AdArgs a = common;
-    a.q = b.qkv + (size_t)z * b.ldq;
-    a.out = b.out + (size_t)z * b.ldo;
+// The caches and positions of the sequences in device memory (llm_batch_desc), read by the kernels when they run:
+// what a captured launch needs, whose arguments cannot change from one replay to the next.
+struct AdBatchDev {
+    const llm_batch_desc *desc;
+    size_t cache_offset; // elements from a sequence's cache pointers to the layer's part of the caches
+};
+
+__device__ __forceinline__ void ad_sequence_caches(const AdBatch &b, const AdBatchDev &, int z, AdArgs &a) {
     a.kc = b.kc[z];
     a.vc = b.vc[z];
     a.pos_host = b.pos[z];
+}
+__device__ __forceinline__ void ad_sequence_caches(const AdBatch &, const AdBatchDev &d, int z, AdArgs &a, int) {
+    a.kc = reinterpret_cast<half_t *>(d.desc->k_cache[z]) + d.cache_offset;
+    a.vc = reinterpret_cast<half_t *>(d.desc->v_cache[z]) + d.cache_offset;
+    int pos = d.desc->pos[z];
+    if (pos > a.max_pos - 1) pos = a.max_pos - 1;
+    a.pos_host = pos < 0 ? 0 : pos;
+}
+
+template <bool DEV>
+__device__ __forceinline__ AdArgs ad_for_sequence(const AdArgs &common, const AdBatch &b, const AdBatchDev &d, int z) {
+    AdArgs a = common;
+    a.q = b.qkv + (size_t)z * b.ldq;
+    a.out = b.out + (size_t)z * b.ldo;
+    if (DEV) ad_sequence_caches(b, d, z, a, 0);
+    else ad_sequence_caches(b, d, z, a);
     a.pos_dev = nullptr;
     if (a.ws_acc) {
         a.ws_acc += (size_t)z * b.ws_floats;
@@ -571,23 +591,24 @@ __device__ __forceinline__ AdArgs ad_for_sequence(const AdArgs &common, const Ad
 }
 
 // every position below 512: the single-span form (dim-split workgroups, direct result)
-template <int HD, int G, int DSN>
-__global__ __launch_bounds__(AD_THREADS) void attn_decode_batch_kernel(const AdArgs common, const AdBatch b) {
+template <int HD, int G, int DSN, bool DEV>
+__global__ __launch_bounds__(AD_THREADS) void attn_decode_batch_kernel(const AdArgs common, const AdBatch b, const AdBatchDev d) {
     __shared__ float sc[G * AD_LS];
     __shared__ __attribute__((aligned(16))) half_t qs[G * HD];
     __shared__ __attribute__((aligned(16))) half_t knew[HD];
     __shared__ __attribute__((aligned(16))) half_t vnew[HD];
     __shared__ float s_m[G], s_l[G];
     __shared__ int s_last;
-    const AdArgs a = ad_for_sequence(common, b, blockIdx.z);
+    AdArgs a = ad_for_sequence<DEV>(common, b, d, blockIdx.z);
+    if (a.pos_host > AD_LS - 1) a.pos_host = AD_LS - 1; // this form serves one span; the host picks it below AD_LS only
     const int y = blockIdx.y;
     attn_decode_body<HD, G, true, HD / DSN, AD_LS>(a, sc, qs, knew, vnew, s_m, s_l, &s_last, a.pos_host, 1, 0,
                                                    y * (HD / DSN), y == 0);
 }
 
-template <int HD, int G>
-__global__ __launch_bounds__(AD_SPAN_THREADS, 4) void attn_span_batch_kernel(const AdArgs common, const AdBatch b) {
-    const AdArgs a = ad_for_sequence(common, b, blockIdx.z);
+template <int HD, int G, bool DEV>
+__global__ __launch_bounds__(AD_SPAN_THREADS, 4) void attn_span_batch_kernel(const AdArgs common, const AdBatch b, const AdBatchDev d) {
+    const AdArgs a = ad_for_sequence<DEV>(common, b, d, blockIdx.z);
     const int span = ad_long_span(a.pos_host + 1, a.span_target);
     const int n_active = (a.pos_host + span) / span;
     const int y = blockIdx.y;
@@ -596,20 +617,27 @@ __global__ __launch_bounds__(AD_SPAN_THREADS, 4) void attn_span_batch_kernel(con
     else attn_span_wave<HD, G, false>(a, a.pos_host, y, blockIdx.x, span);
 }
 
-template <int HD, int G>
-__global__ __launch_bounds__(AD_MERGE_THREADS) void attn_merge_batch_kernel(const AdArgs common, const AdBatch b) {
-    attn_merge_body<HD, G>(ad_for_sequence(common, b, blockIdx.y), blockIdx.x);
+template <int HD, int G, bool DEV>
+__global__ __launch_bounds__(AD_MERGE_THREADS) void attn_merge_batch_kernel(const AdArgs common, const AdBatch b, const AdBatchDev d) {
+    attn_merge_body<HD, G>(ad_for_sequence<DEV>(common, b, d, blockIdx.y), blockIdx.x);
 }
 
+// long_form: < 0 decides from the host's positions in b; with a descriptor in device memory the caller decides
+// (0: every position below AD_LS, 1: the span + merge form) and the span grid covers any position below max_pos.
 template <int HD, int G>
-static int launch_decode_batch(AdArgs a, const AdBatch &b, int B, void *ws, hipStream_t s) {
+static int launch_decode_batch(AdArgs a, const AdBatch &b, const AdBatchDev &d, int long_form, int B, void *ws, hipStream_t s) {
     constexpr int DSN = HD >= 128 ? 4 : 1;
     const int Hq = a.n_kv_heads * G;
-    int max_pos_used = 0;
-    for (int z = 0; z < B; ++z) max_pos_used = b.pos[z] > max_pos_used ? b.pos[z] : max_pos_used;
-    if (max_pos_used < AD_LS) {
+    const bool dev = d.desc != nullptr;
+    if (long_form < 0) {
+        int max_pos_used = 0;
+        for (int z = 0; z < B; ++z) max_pos_used = b.pos[z] > max_pos_used ? b.pos[z] : max_pos_used;
+        long_form = max_pos_used < AD_LS ? 0 : 1;
+    }
+    if (!long_form) {
         a.ws_acc = nullptr;
-        attn_decode_batch_kernel<HD, G, DSN><<<dim3(a.n_kv_heads, DSN, B), dim3(AD_THREADS), 0, s>>>(a, b);
+        if (dev) attn_decode_batch_kernel<HD, G, DSN, true><<<dim3(a.n_kv_heads, DSN, B), dim3(AD_THREADS), 0, s>>>(a, b, d);
+        else attn_decode_batch_kernel<HD, G, DSN, false><<<dim3(a.n_kv_heads, DSN, B), dim3(AD_THREADS), 0, s>>>(a, b, d);
         LLM_LAUNCH_CHECK("attn_decode_batch_kernel");
         return LLM_OK;
     }
@@ -620,14 +648,22 @@ static int launch_decode_batch(AdArgs a, const AdBatch &b, int B, void *ws, hipS
     a.pos_host = 0;
     int rc = ad_long_setup(a, &gy);
     if (rc != LLM_OK) return rc;
+    if (dev) {
+        gy = a.splits; // any position below max_pos
+        attn_span_batch_kernel<HD, G, true><<<dim3(a.n_kv_heads, gy, B), dim3(AD_SPAN_THREADS), 0, s>>>(a, b, d);
+        LLM_LAUNCH_CHECK("attn_span_batch_kernel");
+        attn_merge_batch_kernel<HD, G, true><<<dim3(Hq, B), dim3(AD_MERGE_THREADS), 0, s>>>(a, b, d);
+        LLM_LAUNCH_CHECK("attn_merge_batch_kernel");
+        return LLM_OK;
+    }
     gy = 1;
     for (int z = 0; z < B; ++z) { // the sequence with the most spans sizes the grid (not always the longest one)
         const int n = ad_long_spans(b.pos[z] + 1, a.span_target);
         gy = n > gy ? n : gy;
     }
-    attn_span_batch_kernel<HD, G><<<dim3(a.n_kv_heads, gy, B), dim3(AD_SPAN_THREADS), 0, s>>>(a, b);
+    attn_span_batch_kernel<HD, G, false><<<dim3(a.n_kv_heads, gy, B), dim3(AD_SPAN_THREADS), 0, s>>>(a, b, d);
     LLM_LAUNCH_CHECK("attn_span_batch_kernel");
-    attn_merge_batch_kernel<HD, G><<<dim3(Hq, B), dim3(AD_MERGE_THREADS), 0, s>>>(a, b);
+    attn_merge_batch_kernel<HD, G, false><<<dim3(Hq, B), dim3(AD_MERGE_THREADS), 0, s>>>(a, b, d);
     LLM_LAUNCH_CHECK("attn_merge_batch_kernel");
     return LLM_OK;
 }
@@ -974,8 +1010,9 @@ int llm_attn_decode_rope_batch(const uint16_t *qkv, int ldq, uint16_t *const *k_
     a.max_pos = max_pos;
     const int G = n_heads / n_kv_heads;
     hipStream_t s = (hipStream_t)stream;
+    const AdBatchDev d = {nullptr, 0};
 #define AD_CASE(HD_, G_) \
-    if (head_dim == HD_ && G == G_) return launch_decode_batch<HD_, G_>(a, b, batch, workspace, s);
+    if (head_dim == HD_ && G == G_) return launch_decode_batch<HD_, G_>(a, b, d, -1, batch, workspace, s);
     AD_CASE(128, 4)
     AD_CASE(128, 8)
     AD_CASE(128, 1)
@@ -985,6 +1022,45 @@ int llm_attn_decode_rope_batch(const uint16_t *qkv, int ldq, uint16_t *const *k_
     AD_CASE(32, 1)
 #undef AD_CASE
     llm_set_error("llm_attn_decode_rope_batch: head_dim=%d with group size %d is not built", head_dim, G);
+    return LLM_ERR_INVALID;
+}
+
+int llm_attn_decode_rope_batch_dev(const uint16_t *qkv, int ldq, const llm_batch_desc *desc_dev, size_t cache_offset, int batch,
+                                   int long_form, uint16_t *out, int ldo, const float *table, int n_heads, int n_kv_heads,
+                                   int head_dim, int max_pos, void *workspace, llm_stream_t stream) {
+    LLM_REQUIRE(qkv && desc_dev && out && table && workspace, "llm_attn_decode_rope_batch_dev: null pointer");
+    LLM_REQUIRE(batch >= 1 && batch <= AD_MAX_BATCH && LLM_MAX_BATCH == AD_MAX_BATCH, "llm_attn_decode_rope_batch_dev: batch=%d (1..%d)",
+                batch, AD_MAX_BATCH);
+    LLM_REQUIRE(n_kv_heads > 0 && n_heads % n_kv_heads == 0, "llm_attn_decode_rope_batch_dev: heads %d/%d", n_heads, n_kv_heads);
+    LLM_REQUIRE(max_pos > 0 && max_pos % 64 == 0, "llm_attn_decode_rope_batch_dev: max_pos=%d must be a multiple of 64", max_pos);
+    LLM_REQUIRE(ldq % 8 == 0 && ldq >= (n_heads + 2 * n_kv_heads) * head_dim && ldo >= n_heads * head_dim,
+                "llm_attn_decode_rope_batch_dev: ldq=%d ldo=%d", ldq, ldo);
+    LLM_REQUIRE(aligned16(qkv) && cache_offset % 8 == 0, "llm_attn_decode_rope_batch_dev: qkv and the cache offset must be 16-byte aligned");
+    LLM_REQUIRE(long_form == 0 || long_form == 1, "llm_attn_decode_rope_batch_dev: long_form is 0 or 1");
+    AdBatch b = {};
+    b.qkv = (const half_t *)qkv;
+    b.ldq = ldq;
+    b.out = (half_t *)out;
+    b.ldo = ldo;
+    b.ws_floats = llm_attn_decode_workspace_bytes(n_heads, head_dim) / sizeof(float);
+    const AdBatchDev d = {desc_dev, cache_offset};
+    AdArgs a = {};
+    a.table = table;
+    a.n_kv_heads = n_kv_heads;
+    a.max_pos = max_pos;
+    const int G = n_heads / n_kv_heads;
+    hipStream_t s = (hipStream_t)stream;
+#define AD_CASE(HD_, G_) \
+    if (head_dim == HD_ && G == G_) return launch_decode_batch<HD_, G_>(a, b, d, long_form, batch, workspace, s);
+    AD_CASE(128, 4)
+    AD_CASE(128, 8)
+    AD_CASE(128, 1)
+    AD_CASE(64, 4)
+    AD_CASE(64, 1)
+    AD_CASE(32, 4)
+    AD_CASE(32, 1)
+#undef AD_CASE
+    llm_set_error("llm_attn_decode_rope_batch_dev: head_dim=%d with group size %d is not built", head_dim, G);
     return LLM_ERR_INVALID;
 }
 

@@ -89,6 +89,13 @@ struct Engine {
     llm_half *b_logits = nullptr; // [batch][vocab]
     int32_t *b_ids = nullptr;     // [batch] input ids, then the argmax results
     void *b_ws_attn = nullptr, *b_ws_argmax = nullptr;
+    // the sequences' caches and positions where the kernels of a batched step read them, its pinned mirror, pinned
+    // staging for the ids in and out; one captured step per (batch size, attention form), taken into use once that
+    // combination has run with plain launches
+    llm_batch_desc *b_desc = nullptr, *b_desc_host = nullptr;
+    int32_t *b_ids_host = nullptr;
+    llm_graph_t b_graph[17][2] = {};
+    bool b_ran[17][2] = {};
     llm_event_t ev[4] = {nullptr, nullptr, nullptr, nullptr};
 };
 
@@ -149,6 +156,11 @@ void drop_graph(Engine *e) {
         llm_graph_destroy(e->graph[f]);
         e->graph[f] = nullptr;
     }
+    for (auto &per_batch : e->b_graph)
+        for (llm_graph_t &g : per_batch) {
+            if (g) llm_graph_destroy(g);
+            g = nullptr;
+        }
 }
 
 // The captured decode graphs hold the weight pointers of the model they were captured with.  A call
@@ -466,6 +478,41 @@ int step_one(Engine *e, const Llama3 *m, int token, llm_half *logits_host) {
     return (int)e->h_stage[2];
 }
 
+// One batched decode step on e0's stream from device state: ids in e0->b_ids, caches and positions in e0->b_desc;
+// leaves the greedy ids in e0->b_ids and the logits in e0->b_logits.  Nothing in it depends on host values that
+// change from step to step, so it can be captured.  form: 0 every position below LONG_ATTN_FROM, 1 otherwise.
+void issue_batch_step(Engine *e0, const Llama3 *m, int batch, int form) {
+    const ModelConfig &c = e0->cfg;
+    const int d = c.d_model, hd = c.head_dim, Hq = c.n_heads, Hkv = c.n_kv_heads, F = c.ffn_dim;
+    const int qd = Hq * hd, kvd = Hkv * hd, QKV = e0->qkv_dim;
+    llm_stream_t s = e0->stream;
+    llama3_check(llm_embed_gather(m->embed_tokens->d_fp16_tensor, e0->b_ids, nullptr, e0->x, batch, d, c.vocab, s),
+                 "llm_embed_gather");
+    for (int l = 0; l < c.n_layers; ++l) {
+        const LayerW w = layer_w(m, l);
+        llama3_check(llm_rmsnorm(e0->x, w.in_ln, e0->xn, batch, d, c.rms_eps, s), "llm_rmsnorm");
+        if (w.wk == w.wq + (size_t)qd * d && w.wv == w.wk + (size_t)kvd * d) {
+            llama3_check(llm_linear(e0->xn, d, w.wq, nullptr, 0, e0->qkv, QKV, batch, QKV, d, s), "llm_linear(qkv)");
+        } else {
+            llama3_check(llm_linear(e0->xn, d, w.wq, nullptr, 0, e0->qkv, QKV, batch, qd, d, s), "llm_linear(q)");
+            llama3_check(llm_linear(e0->xn, d, w.wk, nullptr, 0, e0->qkv + qd, QKV, batch, kvd, d, s), "llm_linear(k)");
+            llama3_check(llm_linear(e0->xn, d, w.wv, nullptr, 0, e0->qkv + qd + kvd, QKV, batch, kvd, d, s), "llm_linear(v)");
+        }
+        llama3_check(llm_attn_decode_rope_batch_dev(e0->qkv, QKV, e0->b_desc, (size_t)l * e0->kv_layer_elems, batch, form, e0->attn,
+                                                    qd, e0->rope_table, Hq, Hkv, hd, c.max_pos, e0->b_ws_attn, s),
+                     "llm_attn_decode_rope_batch_dev");
+        llama3_check(llm_linear(e0->attn, qd, w.wo, e0->x, d, e0->x, d, batch, d, qd, s), "llm_linear(o)");
+        llama3_check(llm_rmsnorm(e0->x, w.post_ln, e0->xn, batch, d, c.rms_eps, s), "llm_rmsnorm");
+        llama3_check(llm_linear_swiglu(e0->xn, d, w.wg, w.wu, e0->ffn, F, batch, F, d, s), "llm_linear_swiglu");
+        llama3_check(llm_linear(e0->ffn, F, w.wd, e0->x, d, e0->x, d, batch, d, F, s), "llm_linear(down)");
+    }
+    llama3_check(llm_rmsnorm(e0->x, m->norm->d_fp16_tensor, e0->xn, batch, d, c.rms_eps, s), "llm_rmsnorm");
+    llama3_check(llm_linear(e0->xn, d, m->lm_head->d_fp16_tensor, nullptr, 0, e0->b_logits, c.vocab, batch, c.vocab, d, s),
+                 "llm_linear(lm_head)");
+    llama3_check(llm_argmax_f16_rows(e0->b_logits, c.vocab, batch, c.vocab, e0->b_ids, e0->b_ws_argmax, s),
+                 "llm_argmax_f16_rows");
+}
+
 } // namespace
 
 // ---------------------------------------------------------------------------
@@ -563,11 +610,13 @@ extern "C" void free_cache(CudaCache *C) {
         drop_graph(e);
         void *bufs[] = {e->x, e->xn, e->qkv, e->attn, e->ffn, e->logits, e->kc, e->vc, e->rope_table,
                         e->d_tokens, e->d_pos, e->d_token, e->ao_ring, e->ws_attn, e->ws_lm, e->trace_dev, e->inject_dev,
-                        e->b_logits, e->b_ids, e->b_ws_attn, e->b_ws_argmax};
+                        e->b_logits, e->b_ids, e->b_ws_attn, e->b_ws_argmax, e->b_desc};
         for (void *b : bufs) llm_free(b);
         for (auto ev : e->ev) llm_event_destroy(ev);
         llm_stream_destroy(e->stream);
         llm_free_host(e->h_stage);
+        if (e->b_desc_host) llm_free_host(e->b_desc_host);
+        if (e->b_ids_host) llm_free_host(e->b_ids_host);
         if (e->h_select) llm_free_host(e->h_select);
         if (e->d_select) llm_free(e->d_select);
         if (e->d_exp_table) llm_free(e->d_exp_table);
@@ -681,8 +730,7 @@ extern "C" void llama3_decode_batch(Llama3 *m, CudaCache *const *caches, const i
     Engine *e0 = eng(caches[0]);
     const ModelConfig &c = e0->cfg;
     bind_model(e0, m);
-    const int d = c.d_model, hd = c.head_dim, Hq = c.n_heads, Hkv = c.n_kv_heads, F = c.ffn_dim;
-    const int qd = Hq * hd, kvd = Hkv * hd, QKV = e0->qkv_dim;
+    const int d = c.d_model, hd = c.head_dim, Hq = c.n_heads;
     llm_stream_t s = e0->stream;
     Engine *es[16];
     int pos[16];
@@ -691,7 +739,8 @@ extern "C" void llama3_decode_batch(Llama3 *m, CudaCache *const *caches, const i
         for (int a = 0; a < b; ++a)
             if (es[a] == es[b]) llama3_fail("llama3_decode_batch: sequence %d and %d share a cache", a, b);
         const ModelConfig &cb = es[b]->cfg;
-        if (cb.max_pos != c.max_pos || cb.d_model != d || cb.n_layers != c.n_layers || cb.vocab != c.vocab)
+        if (cb.max_pos != c.max_pos || cb.d_model != d || cb.n_layers != c.n_layers || cb.vocab != c.vocab ||
+            cb.n_kv_heads != c.n_kv_heads || cb.head_dim != c.head_dim)
             llama3_fail("llama3_decode_batch: cache %d has a different configuration", b);
         if (es[b]->pos + 1 > c.max_pos) llama3_fail("sequence of %d tokens exceeds max_pos %d", es[b]->pos + 1, c.max_pos);
         if (tokens[b] < 0 || tokens[b] >= c.vocab) llama3_fail("token id %d outside the vocabulary", tokens[b]);
@@ -710,44 +759,44 @@ extern "C" void llama3_decode_batch(Llama3 *m, CudaCache *const *caches, const i
         e0->b_ws_attn = dmalloc<char>(wsb * 16, "llm_malloc(batch attention workspace)");
         llama3_check(llm_fill_zero(e0->b_ws_attn, wsb * 16, s), "zero workspace");
         e0->b_ws_argmax = dmalloc<char>((size_t)16 * 1024 * 8, "llm_malloc(batch argmax candidates)");
+        if (!e0->b_desc) {
+            e0->b_desc = dmalloc<llm_batch_desc>(1, "llm_malloc(batch descriptor)");
+            void *hp = nullptr;
+            llama3_check(llm_malloc_host(&hp, sizeof(llm_batch_desc)), "llm_malloc_host(batch descriptor)");
+            e0->b_desc_host = (llm_batch_desc *)hp;
+            llama3_check(llm_malloc_host(&hp, sizeof(int32_t) * 16), "llm_malloc_host(batch ids)");
+            e0->b_ids_host = (int32_t *)hp;
+        }
         e0->batch_cap = 16;
     }
-    llama3_check(llm_memcpy_h2d(e0->b_ids, tokens, sizeof(int32_t) * (size_t)batch, s), "H2D ids");
-    llama3_check(llm_embed_gather(m->embed_tokens->d_fp16_tensor, e0->b_ids, nullptr, e0->x, batch, d, c.vocab, s),
-                 "llm_embed_gather");
-    for (int l = 0; l < c.n_layers; ++l) {
-        const LayerW w = layer_w(m, l);
-        uint16_t *kcs[16], *vcs[16];
-        for (int b = 0; b < batch; ++b) {
-            kcs[b] = es[b]->kc + (size_t)l * es[b]->kv_layer_elems;
-            vcs[b] = es[b]->vc + (size_t)l * es[b]->kv_layer_elems;
-        }
-        llama3_check(llm_rmsnorm(e0->x, w.in_ln, e0->xn, batch, d, c.rms_eps, s), "llm_rmsnorm");
-        if (w.wk == w.wq + (size_t)qd * d && w.wv == w.wk + (size_t)kvd * d) {
-            llama3_check(llm_linear(e0->xn, d, w.wq, nullptr, 0, e0->qkv, QKV, batch, QKV, d, s), "llm_linear(qkv)");
-        } else {
-            llama3_check(llm_linear(e0->xn, d, w.wq, nullptr, 0, e0->qkv, QKV, batch, qd, d, s), "llm_linear(q)");
-            llama3_check(llm_linear(e0->xn, d, w.wk, nullptr, 0, e0->qkv + qd, QKV, batch, kvd, d, s), "llm_linear(k)");
-            llama3_check(llm_linear(e0->xn, d, w.wv, nullptr, 0, e0->qkv + qd + kvd, QKV, batch, kvd, d, s), "llm_linear(v)");
-        }
-        llama3_check(llm_attn_decode_rope_batch(e0->qkv, QKV, kcs, vcs, pos, batch, e0->attn, qd, e0->rope_table, Hq, Hkv,
-                                                hd, c.max_pos, e0->b_ws_attn, s),
-                     "llm_attn_decode_rope_batch");
-        llama3_check(llm_linear(e0->attn, qd, w.wo, e0->x, d, e0->x, d, batch, d, qd, s), "llm_linear(o)");
-        llama3_check(llm_rmsnorm(e0->x, w.post_ln, e0->xn, batch, d, c.rms_eps, s), "llm_rmsnorm");
-        llama3_check(llm_linear_swiglu(e0->xn, d, w.wg, w.wu, e0->ffn, F, batch, F, d, s), "llm_linear_swiglu");
-        llama3_check(llm_linear(e0->ffn, F, w.wd, e0->x, d, e0->x, d, batch, d, F, s), "llm_linear(down)");
+    // ids, caches and positions to the device through pinned staging, in stream order in front of the step
+    bool long_form = false;
+    for (int b = 0; b < batch; ++b) {
+        e0->b_ids_host[b] = tokens[b];
+        e0->b_desc_host->k_cache[b] = es[b]->kc;
+        e0->b_desc_host->v_cache[b] = es[b]->vc;
+        e0->b_desc_host->pos[b] = pos[b];
+        long_form = long_form || pos[b] >= LONG_ATTN_FROM;
     }
-    llama3_check(llm_rmsnorm(e0->x, m->norm->d_fp16_tensor, e0->xn, batch, d, c.rms_eps, s), "llm_rmsnorm");
-    llama3_check(llm_linear(e0->xn, d, m->lm_head->d_fp16_tensor, nullptr, 0, e0->b_logits, c.vocab, batch, c.vocab, d, s),
-                 "llm_linear(lm_head)");
-    llama3_check(llm_argmax_f16_rows(e0->b_logits, c.vocab, batch, c.vocab, e0->b_ids, e0->b_ws_argmax, s),
-                 "llm_argmax_f16_rows");
-    int32_t out[16];
-    llama3_check(llm_memcpy_d2h(out, e0->b_ids, sizeof(int32_t) * (size_t)batch, s), "D2H tokens");
+    llama3_check(llm_memcpy_h2d(e0->b_ids, e0->b_ids_host, sizeof(int32_t) * (size_t)batch, s), "H2D ids");
+    llama3_check(llm_memcpy_h2d(e0->b_desc, e0->b_desc_host, sizeof(llm_batch_desc), s), "H2D batch descriptor");
+    const int form = long_form ? 1 : 0;
+    if (e0->use_graph && e0->b_ran[batch][form]) {
+        llm_graph_t &g = e0->b_graph[batch][form];
+        if (!g) {
+            llama3_check(llm_graph_capture_begin(s), "graph capture begin");
+            issue_batch_step(e0, m, batch, form);
+            llama3_check(llm_graph_capture_end(s, &g), "graph capture end");
+        }
+        llama3_check(llm_graph_launch(g, s), "graph launch");
+    } else {
+        issue_batch_step(e0, m, batch, form);
+        e0->b_ran[batch][form] = true;
+    }
+    llama3_check(llm_memcpy_d2h(e0->b_ids_host, e0->b_ids, sizeof(int32_t) * (size_t)batch, s), "D2H tokens");
     llama3_check(llm_stream_sync(s), "stream sync");
     for (int b = 0; b < batch; ++b) {
-        next_tokens[b] = (int)out[b];
+        next_tokens[b] = (int)e0->b_ids_host[b];
         es[b]->tokens.push_back(tokens[b]);
         es[b]->pos += 1;
         es[b]->dev_pos_valid = false; // the batched step keeps no per-cache position on the device

@@ -272,16 +272,19 @@ def test_driver_chat_turn_with_tokenizer(gpu, tmp_path):
     model.close()
 
 
+@pytest.mark.parametrize("use_graph", [False, True])
 @pytest.mark.parametrize("lens", [[5], [7, 40, 3, 21], [500, 20, 515, 9, 64, 130, 2, 33, 77, 5, 6, 90, 100, 250, 11, 12]])
-def test_batched_decode_matches_independent_sequences(gpu, lens):
+def test_batched_decode_matches_independent_sequences(gpu, lens, use_graph):
     """llama3_decode_batch: sequences of different lengths (one crossing 512 cached positions, which switches
-    the whole launch to the span + merge attention) advance together; each must follow its own oracle."""
+    the whole launch to the span + merge attention) advance together; each must follow its own oracle.  With
+    graphs the first step of a (batch size, attention form) runs as plain launches and every later one replays
+    one capture, whose kernels read the caches and positions from device memory."""
     cfg = gpu.engine.config("tiny", max_pos=1024)
     model = gpu.engine.Model.seeded(cfg, 17)
     w = H.oracle_weights(model)
     model.to_device()
     B = len(lens)
-    engines = [gpu.engine.Engine(model, cfg, use_graph=False) for _ in range(B)]
+    engines = [gpu.engine.Engine(model, cfg, use_graph=use_graph) for _ in range(B)]
     oracles = [orc.Model(H.cfg_dict(cfg), w, orc.ORC_REF16) for _ in range(B)]
     cur = []
     for b, n in enumerate(lens):
@@ -313,6 +316,36 @@ def test_batched_decode_matches_independent_sequences(gpu, lens):
         e.close()
     for o in oracles:
         o.close()
+    model.close()
+
+
+def test_batched_decode_graph_replays_equal_plain_launches(gpu):
+    """The captured batched step against plain launches at the 8B layer shapes (2 layers): the same ids and the
+    same logits bit for bit on every step, with the set of caches changing between replays (the captured kernels
+    read cache pointers and positions from device memory) and a single-sequence step of one member in between."""
+    cfg = gpu.engine.config("8b", n_layers=2, max_pos=640)
+    model = gpu.engine.Model.seeded(cfg, 23).to_device()
+    lens = [30, 7, 500, 64]
+    runs = {}
+    for use_graph in (False, True):
+        engines = [gpu.engine.Engine(model, cfg, use_graph=use_graph) for _ in lens]
+        cur = [engines[b].prefill(gpu.engine.seeded_tokens(300 + b, n, cfg.vocab))[0] for b, n in enumerate(lens)]
+        trace = []
+        for step in range(16):                      # sequence 2 crosses position 512 at step 12: the long form takes over
+            order = list(range(4)) if step % 3 else [0, 3, 2, 1]   # caches[0] stays, the others change places
+            nxt = gpu.engine.Engine.decode_batch([engines[i] for i in order], [cur[i] for i in order])
+            for slot, i in enumerate(order):
+                cur[i] = nxt[slot]
+                trace.append((step, i, nxt[slot], engines[0].batch_logits(slot).copy()))
+            if step == 5:                           # eager work of another kind between two replays
+                cur[1] = engines[1].decode(cur[1])[0]
+                trace.append((step, 1, cur[1], engines[1].logits()))
+        runs[use_graph] = trace
+        for e in engines:
+            e.close()
+    assert len(runs[False]) == len(runs[True])
+    for a, b in zip(runs[False], runs[True]):
+        assert a[:3] == b[:3] and np.array_equal(a[3], b[3]), a[:3]
     model.close()
 
 
