@@ -15,6 +15,8 @@
 #include <string>
 #include <vector>
 
+#include <sys/stat.h>
+
 #include "common/fail.h"
 #include "llama3_host.h"
 #include "safetensor/json.h"
@@ -26,35 +28,42 @@ static thread_local int g_decode_size = 128256;
 
 extern "C" {
 
-// tokenizer.cu:231-245
+// tokenizer.cu:231-245: size of a file in bytes, -1 (and a message through perror) when it cannot be examined
 long _get_file_size(const char *filename) {
-    FILE *file = fopen(filename, "rb");
-    if (file == NULL) {
+    struct stat st;
+    if (stat(filename, &st) != 0) {
         perror("Failed to open file");
         return -1;
     }
-    fseek(file, 0, SEEK_END);
-    long size = ftell(file);
-    fclose(file);
-    return size;
+    return (long)st.st_size;
 }
 
-// tokenizer.cu:200-229
+// tokenizer.cu:200-229: the whole file as one NUL-terminated string that the caller frees.  One open: the size
+// comes from the descriptor that is then read, so a file replaced between the two steps cannot overrun.
 char *read_tokenizer_json(Llama3Tokenizer *tokenizer, const char *filename) {
     (void)tokenizer;
-    long size = _get_file_size(filename);
-    if (size == -1) llama3_fail("Could not determine file size");
-    char *buffer = (char *)malloc((size_t)size + 1);
-    if (buffer == NULL) llama3_fail("Memory allocation failed for buffer");
-    FILE *fp = fopen(filename, "r");
-    if (fp == NULL) {
-        free(buffer);
-        llama3_fail("Could not open file %s", filename);
+    FILE *in = fopen(filename, "rb");
+    struct stat st;
+    if (in == NULL || fstat(fileno(in), &st) != 0) { // the reference's two messages for a file it cannot size
+        perror("Failed to open file");
+        if (in) fclose(in);
+        llama3_fail("Could not determine file size");
     }
-    size_t got = fread(buffer, 1, (size_t)size, fp);
-    buffer[got] = '\0';
-    fclose(fp);
-    return buffer;
+    const size_t want = (size_t)st.st_size;
+    char *text = (char *)malloc(want + 1);
+    if (text == NULL) {
+        fclose(in);
+        llama3_fail("Memory allocation failed for buffer");
+    }
+    size_t have = 0;
+    while (have < want) {
+        const size_t n = fread(text + have, 1, want - have, in);
+        if (n == 0) break;
+        have += n;
+    }
+    fclose(in);
+    text[have] = '\0';
+    return text;
 }
 
 // ---- the byte trie -------------------------------------------------------------------------------------
