@@ -153,6 +153,26 @@ def test_linear_skinny(gpu, name, T):
     assert e <= TIGHT
 
 
+@pytest.mark.parametrize("tiles", [30, 100, 140, 256 + 40, 256 + 128, 256 + 200, 2 * 256 + 31])
+@pytest.mark.parametrize("T", [2, 5, 16])
+def test_skinny_tile_counts_around_the_cu_count(gpu, tiles, T):
+    """The 2..16-row kernel walks persistently over 16-column tiles, one workgroup per CU: tile counts below, at
+    and above multiples of the CU count (last rounds that are nearly empty, half full, nearly full) all write every
+    output column once and match the oracle, with and without the residual and through the SwiGLU epilogue."""
+    K, N = 1024, 16 * tiles
+    rng = np.random.default_rng(tiles * 31 + T)
+    x = H.bits(rng.standard_normal((T, K)))
+    w = H.bits(0.05 * rng.standard_normal((N, K), dtype=np.float32))
+    w2 = H.bits(0.05 * rng.standard_normal((N, K), dtype=np.float32))
+    res = H.bits(rng.standard_normal((T, N)))
+    say("skinny tiles", tiles, T)
+    got = gpu.ops.linear(x, w, residual=res)
+    assert H.mixed_err(got, orc.add(orc.linear(x, w), res)) <= TIGHT
+    assert np.array_equal(gpu.ops.linear(x, w, residual=res, inplace=True), got)   # out == residual, as the engine calls it
+    assert H.mixed_err(gpu.ops.linear(x, w), orc.linear(x, w)) <= TIGHT
+    assert H.mixed_err(gpu.ops.linear_swiglu(x, w, w2), orc.linear_swiglu(x, w, w2)) <= TIGHT
+
+
 @pytest.mark.parametrize("T", [1, 4, 16])
 def test_linear_residual_epilogue(gpu, T):
     K, N = 4096, 4096
