@@ -112,6 +112,11 @@ int llm_rope(uint16_t *buf_dev, int T, int n_heads, int head_dim, int row_stride
 int llm_rope_kv_append(uint16_t *qkv_dev, uint16_t *k_cache_dev, uint16_t *v_cache_dev, int T,
                        int n_heads, int n_kv_heads, int head_dim, int pos0, const int32_t *pos_dev,
                        const float *table_dev, int max_pos, llm_stream_t stream);
+/* The same without the pass over Q: K is rotated into the K cache and V stored into the V cache, the queries in qkv
+ * stay as the projection left them -- for a prompt pass whose attention rotates the queries itself
+ * (llm_attn_prefill_rope_q).  At least 16 rows, positions known on the host. */
+int llm_rope_k_append(uint16_t *qkv_dev, uint16_t *k_cache_dev, uint16_t *v_cache_dev, int T, int n_heads,
+                      int n_kv_heads, int head_dim, int pos0, const float *table_dev, int max_pos, llm_stream_t stream);
 
 /* ---- projections -------------------------------------------------------------- */
 /* Replaces kernel_standard_tiled_gemm and its launchers compute_qkv_tensors,
@@ -272,6 +277,16 @@ int llm_attn_decode_rope_batch_dev(const uint16_t *qkv_dev, int ldq, const llm_b
 int llm_attn_prefill(const uint16_t *q_dev, int ldq, const uint16_t *k_cache_dev,
                      const uint16_t *v_cache_dev, uint16_t *out_dev, int ldo, int T, int pos0,
                      int n_heads, int n_kv_heads, int head_dim, int max_pos, llm_stream_t stream);
+/* llm_attn_prefill on queries that have not been rotated yet (rope_scaling of Q, src/inference/inference.cu:621-695,
+ * folded into the attention): every wavefront rotates the query fragments it has just loaded by the angles of
+ * their rows' positions (table_dev as for llm_rope) -- the arithmetic of llm_rope on the same elements, so the
+ * result has the bits of llm_rope on Q followed by llm_attn_prefill, and Q is not read and written once more
+ * (134 MB per layer of an 8192-token pass).  Served by the pipelined kernel only: head size 128, four query heads
+ * per KV head, at least 64 rows (llm_attn_prefill_rope_q_supported says 1); other shapes return LLM_ERR_INVALID. */
+int llm_attn_prefill_rope_q_supported(int T, int n_heads, int n_kv_heads, int head_dim, int max_pos);
+int llm_attn_prefill_rope_q(const uint16_t *q_dev, int ldq, const uint16_t *k_cache_dev, const uint16_t *v_cache_dev,
+                            uint16_t *out_dev, int ldo, int T, int pos0, const float *table_dev, int n_heads,
+                            int n_kv_heads, int head_dim, int max_pos, llm_stream_t stream);
 
 /* ---- sampler candidates --------------------------------------------------------------------------- */
 /* Device half of sample_next_token (src/inference/inference.cu:1030-1161): what temperature_softmax's

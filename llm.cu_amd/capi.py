@@ -112,6 +112,7 @@ HIP_ABI = {
     "llm_rope_table_host": (_i, [_vp, _i, _i, C.c_float]),
     "llm_rope": (_i, [_vp, _i, _i, _i, _i, _i, _vp, _vp, _i, _vp]),
     "llm_rope_kv_append": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _vp, _i, _vp]),
+    "llm_rope_k_append": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _i, _vp]),
     "llm_linear": (_i, [_vp, _i, _vp, _vp, _i, _vp, _i, _i, _i, _i, _vp]),
     "llm_linear_unsplit_fallbacks": (C.c_long, []),
     "llm_linear_swiglu": (_i, [_vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
@@ -137,6 +138,8 @@ HIP_ABI = {
     "llm_attn_decode_noalloc_max_bytes": (_sz, []),
     "llm_attn_decode_noalloc": (_i, [_vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _i, _vp]),
     "llm_attn_prefill": (_i, [_vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp]),
+    "llm_attn_prefill_rope_q_supported": (_i, [_i, _i, _i, _i, _i]),
+    "llm_attn_prefill_rope_q": (_i, [_vp, _i, _vp, _vp, _vp, _i, _i, _i, _vp, _i, _i, _i, _i, _vp]),
     "llm_lmhead_workspace_bytes": (_sz, [_i]),
     "llm_lmhead_argmax": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp, _vp]),
     "llm_argmax_f16": (_i, [_vp, _i, _vp, _vp, _vp]),

@@ -361,12 +361,16 @@ __global__ __launch_bounds__(G *AP_QT * 64) void attn_prefill_kernel(const half_
 typedef uint32_t ap_u4_t __attribute__((ext_vector_type(4)));
 typedef uint32_t ap_u8_t __attribute__((ext_vector_type(8)));
 
-template <int G>
+template <int G, bool ROPE_Q>
 __global__ __launch_bounds__(G * 128, 1) void attn_prefill_pipe_kernel(const half_t *__restrict__ q, int ldq,
                                                                        const half_t *__restrict__ kc,
                                                                        const half_t *__restrict__ vc,
                                                                        half_t *__restrict__ out, int ldo, int T,
-                                                                       int pos0, int max_pos) {
+                                                                       int pos0, int max_pos,
+                                                                       const float *__restrict__ table) {
+    // ROPE_Q: q holds the projection as stored; every wavefront rotates its own query fragments by the angles of their
+    // positions (table: [max_pos][64][2], as llm_rope uses it) right after loading them -- the arithmetic of the
+    // RoPE kernel on the same elements, so the same bits, without a pass over Q in memory.
     static_assert(G == 4, "eight wavefronts, two per SIMD");
     constexpr int HD = 128, NW = 2 * G, THREADS = NW * 64;
     constexpr int LPT = 32 / NW;            // tile-load instructions per wavefront and tile
@@ -394,6 +398,12 @@ __global__ __launch_bounds__(G * 128, 1) void attn_prefill_pipe_kernel(const hal
     half8_t qf[8];
 #pragma unroll
     for (int ks = 0; ks < 8; ++ks) qf[ks] = load8(q + (size_t)qrow * ldq + (size_t)head * HD + 16 * ks + 8 * hb);
+    if (ROPE_Q) { // lane (n, hb) holds dims 16 ks + 8 hb .. + 7 of its row: pairs 8 ks + 4 hb .. + 3
+        const int rp = qpos < max_pos ? qpos : max_pos - 1;
+        const float *cs = table + ((size_t)rp * (HD / 2) + 4 * hb) * 2;
+#pragma unroll
+        for (int ks = 0; ks < 8; ++ks) qf[ks] = rope_rotate8(qf[ks], cs + 16 * ks);
+    }
 
     // tile loads straight into LDS: wave instruction i' = wave + NW t covers 1 KB = 4 K rows or 8 V^T rows; lane l
     // writes 16 bytes at 16 l and fetches the 16-byte chunk of its row that the swizzle puts there
@@ -622,15 +632,16 @@ __global__ __launch_bounds__(G * 128, 1) void attn_prefill_pipe_kernel(const hal
     }
 }
 
+template <bool ROPE_Q>
 static int launch_prefill_pipe(const half_t *q, int ldq, const half_t *kc, const half_t *vc, half_t *out, int ldo, int T,
-                               int pos0, int n_kv_heads, int max_pos, hipStream_t s) {
+                               int pos0, int n_kv_heads, int max_pos, const float *table, hipStream_t s) {
     dim3 grid(n_kv_heads, (T + 63) / 64);
     const size_t smem = 8 * 64 * 128 * sizeof(half_t); // four stages of a K and a V^T tile
-    auto kern = attn_prefill_pipe_kernel<4>;
+    auto kern = attn_prefill_pipe_kernel<4, ROPE_Q>;
     static std::atomic<uint64_t> attr_done{0};
     int rc = llm_ensure_max_smem((const void *)kern, smem, attr_done);
     if (rc != LLM_OK) return rc;
-    kern<<<grid, dim3(512), smem, s>>>(q, ldq, kc, vc, out, ldo, T, pos0, max_pos);
+    kern<<<grid, dim3(512), smem, s>>>(q, ldq, kc, vc, out, ldo, T, pos0, max_pos, table);
     LLM_LAUNCH_CHECK("attn_prefill_pipe_kernel");
     return LLM_OK;
 }
@@ -672,7 +683,7 @@ extern "C" int llm_attn_prefill(const uint16_t *q, int ldq, const uint16_t *kc, 
     half_t *op = (half_t *)out;
     // the pipelined kernel addresses one KV head's cache through a 32-bit buffer descriptor
     if (head_dim == 128 && G == 4 && T >= AP_PIPE_MIN_ROWS && (size_t)max_pos * 128 * sizeof(half_t) < (1ull << 31))
-        return launch_prefill_pipe(qp, ldq, kp, vp, op, ldo, T, pos0, n_kv_heads, max_pos, s);
+        return launch_prefill_pipe<false>(qp, ldq, kp, vp, op, ldo, T, pos0, n_kv_heads, max_pos, nullptr, s);
 #define AP_CASE(HD_, G_)                                                                        \
     if (head_dim == HD_ && G == G_)                                                             \
         return launch_prefill<HD_, G_>(qp, ldq, kp, vp, op, ldo, T, pos0, n_kv_heads, max_pos, s);
@@ -686,4 +697,31 @@ extern "C" int llm_attn_prefill(const uint16_t *q, int ldq, const uint16_t *kc, 
 #undef AP_CASE
     llm_set_error("llm_attn_prefill: head_dim=%d with group size %d is not built", head_dim, G);
     return LLM_ERR_INVALID;
+}
+
+// The shapes the pipelined kernel serves: the only ones for which the attention rotates the queries itself.
+static bool prefill_pipe_shape(int T, int n_heads, int n_kv_heads, int head_dim, int max_pos) {
+    return n_kv_heads > 0 && n_heads == 4 * n_kv_heads && head_dim == 128 && T >= AP_PIPE_MIN_ROWS &&
+           (size_t)max_pos * 128 * sizeof(half_t) < (1ull << 31);
+}
+
+extern "C" int llm_attn_prefill_rope_q_supported(int T, int n_heads, int n_kv_heads, int head_dim, int max_pos) {
+    return prefill_pipe_shape(T, n_heads, n_kv_heads, head_dim, max_pos) ? 1 : 0;
+}
+
+extern "C" int llm_attn_prefill_rope_q(const uint16_t *q, int ldq, const uint16_t *kc, const uint16_t *vc, uint16_t *out, int ldo,
+                                       int T, int pos0, const float *table, int n_heads, int n_kv_heads, int head_dim,
+                                       int max_pos, llm_stream_t stream) {
+    LLM_REQUIRE(q && kc && vc && out && table, "llm_attn_prefill_rope_q: null pointer");
+    LLM_REQUIRE(prefill_pipe_shape(T, n_heads, n_kv_heads, head_dim, max_pos),
+                "llm_attn_prefill_rope_q: %d rows, heads %d/%d of %d are not covered (llm_attn_prefill_rope_q_supported)", T, n_heads,
+                n_kv_heads, head_dim);
+    LLM_REQUIRE(pos0 >= 0 && pos0 + T <= max_pos, "llm_attn_prefill_rope_q: rows %d..%d of %d", pos0, pos0 + T, max_pos);
+    LLM_REQUIRE(max_pos % 64 == 0, "llm_attn_prefill_rope_q: max_pos=%d must be a multiple of 64", max_pos);
+    LLM_REQUIRE(ldq % 8 == 0 && ldq >= n_heads * head_dim && ldo % 4 == 0 && ldo >= n_heads * head_dim,
+                "llm_attn_prefill_rope_q: ldq=%d ldo=%d", ldq, ldo);
+    LLM_REQUIRE(aligned16(q) && aligned16(kc) && aligned16(vc) && aligned16(table) && ((uintptr_t)out & 7u) == 0,
+                "llm_attn_prefill_rope_q: pointers must be 16-byte aligned");
+    return launch_prefill_pipe<true>((const half_t *)q, ldq, (const half_t *)kc, (const half_t *)vc, (half_t *)out, ldo, T, pos0,
+                                     n_kv_heads, max_pos, table, (hipStream_t)stream);
 }

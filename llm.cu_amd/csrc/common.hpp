@@ -145,6 +145,21 @@ __device__ __forceinline__ half8_t load8_nt(const half_t *p) {
 }
 __device__ __forceinline__ void store8(half_t *p, half8_t v) { *reinterpret_cast<half8_t *>(p) = v; }
 
+// RoPE of four adjacent pairs (8 halves): (e, o) -> (c e - s o, s e + c o) with unfused multiplies (the device code
+// is compiled with -ffp-contract=off), each result rounded to fp16.  cs: the four (cos, sin) pairs of the position.
+__device__ __forceinline__ half8_t rope_rotate8(half8_t v, const float *__restrict__ cs) {
+    half8_t o;
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+        const float c = cs[2 * p], s = cs[2 * p + 1];
+        const float e = (float)v[2 * p], od = (float)v[2 * p + 1];
+        const float ce = c * e, so = s * od, se = s * e, co = c * od;
+        o[2 * p] = (half_t)(ce - so);
+        o[2 * p + 1] = (half_t)(se + co);
+    }
+    return o;
+}
+
 // fp16 result with an optional residual: the reference stores the projection
 // as fp16 and then adds the fp16 residual in fp32 (two roundings).
 __device__ __forceinline__ half_t finish(float acc, const half_t *res) {

@@ -110,19 +110,7 @@ __global__ __launch_bounds__(THREADS) void rmsnorm_kernel(const half_t *x, // ma
 // e' = c*e - s*o, o' = s*e + c*o with unfused multiplies (this file is
 // compiled with -ffp-contract=off).
 // ---------------------------------------------------------------------------
-__device__ __forceinline__ half8_t rotate8(half8_t v, const float *__restrict__ cs) {
-    // cs: 4 consecutive (cos, sin) pairs
-    half8_t o;
-#pragma unroll
-    for (int p = 0; p < 4; ++p) {
-        float c = cs[2 * p], s = cs[2 * p + 1];
-        float e = (float)v[2 * p], od = (float)v[2 * p + 1];
-        float ce = c * e, so = s * od, se = s * e, co = c * od;
-        o[2 * p] = (half_t)(ce - so);
-        o[2 * p + 1] = (half_t)(se + co);
-    }
-    return o;
-}
+__device__ __forceinline__ half8_t rotate8(half8_t v, const float *__restrict__ cs) { return rope_rotate8(v, cs); }
 
 __global__ __launch_bounds__(256) void rope_kernel(half_t *__restrict__ buf, int n_heads, int head_dim,
                                                    int row_stride, int pos0,
@@ -231,11 +219,12 @@ __global__ __launch_bounds__(256) void rope_qk_append_kernel(half_t *__restrict_
                                                              half_t *__restrict__ kc, int n_heads,
                                                              int n_kv_heads, int head_dim, int pos0,
                                                              const float *__restrict__ table,
-                                                             int max_pos) {
+                                                             int max_pos, int c_begin) {
+    // c_begin: 0, or the width of Q when the queries stay as they are (the attention kernel rotates them itself)
     const int t = blockIdx.y;
     const int qd = n_heads * head_dim, kvd = n_kv_heads * head_dim;
     const int width = qd + 2 * kvd;
-    const int c = (blockIdx.x * blockDim.x + threadIdx.x) * 8;
+    const int c = c_begin + (blockIdx.x * blockDim.x + threadIdx.x) * 8;
     if (c >= qd + kvd) return;
     int pos = pos0 + t;
     if (pos >= max_pos) pos = max_pos - 1;
@@ -354,9 +343,9 @@ int llm_rope(uint16_t *buf, int T, int n_heads, int head_dim, int row_stride, in
     return LLM_OK;
 }
 
-int llm_rope_kv_append(uint16_t *qkv, uint16_t *kc, uint16_t *vc, int T, int n_heads, int n_kv_heads,
-                       int head_dim, int pos0, const int32_t *pos_dev, const float *table, int max_pos,
-                       llm_stream_t stream) {
+static int rope_kv_append(uint16_t *qkv, uint16_t *kc, uint16_t *vc, int T, int n_heads, int n_kv_heads, int head_dim,
+                          int pos0, const int32_t *pos_dev, const float *table, int max_pos, bool keep_q,
+                          llm_stream_t stream) {
     LLM_REQUIRE(qkv && kc && vc && table, "llm_rope_kv_append: null pointer");
     LLM_REQUIRE(T >= 0 && n_heads > 0 && n_kv_heads > 0 && head_dim >= 8 && head_dim % 8 == 0,
                 "llm_rope_kv_append: bad shape");
@@ -366,15 +355,17 @@ int llm_rope_kv_append(uint16_t *qkv, uint16_t *kc, uint16_t *vc, int T, int n_h
     if (T == 0) return LLM_OK;
     hipStream_t s = (hipStream_t)stream;
     const int qd = n_heads * head_dim, kvd = n_kv_heads * head_dim;
+    LLM_REQUIRE(!keep_q || (T >= 16 && !pos_dev), "llm_rope_k_append: at least 16 rows at host-known positions");
     if (T < 16 || pos_dev) {
         dim3 grid(((qd + 2 * kvd) / 8 + 255) / 256, T);
         rope_kv_append_kernel<<<grid, dim3(256), 0, s>>>((half_t *)qkv, (half_t *)kc, (half_t *)vc, n_heads,
                                                          n_kv_heads, head_dim, pos0, pos_dev, table, max_pos);
         LLM_LAUNCH_CHECK("rope_kv_append_kernel");
     } else {
-        dim3 grid(((qd + kvd) / 8 + 255) / 256, T);
+        const int c_begin = keep_q ? qd : 0;
+        dim3 grid(((qd + kvd - c_begin) / 8 + 255) / 256, T);
         rope_qk_append_kernel<<<grid, dim3(256), 0, s>>>((half_t *)qkv, (half_t *)kc, n_heads, n_kv_heads, head_dim,
-                                                         pos0, table, max_pos);
+                                                         pos0, table, max_pos, c_begin);
         LLM_LAUNCH_CHECK("rope_qk_append_kernel");
         dim3 gv((T + 63) / 64, (kvd + 63) / 64);
         v_append_transpose_kernel<<<gv, dim3(256), 0, s>>>((const half_t *)qkv, (half_t *)vc, T, n_heads, n_kv_heads,
@@ -382,6 +373,16 @@ int llm_rope_kv_append(uint16_t *qkv, uint16_t *kc, uint16_t *vc, int T, int n_h
         LLM_LAUNCH_CHECK("v_append_transpose_kernel");
     }
     return LLM_OK;
+}
+
+int llm_rope_kv_append(uint16_t *qkv, uint16_t *kc, uint16_t *vc, int T, int n_heads, int n_kv_heads, int head_dim,
+                       int pos0, const int32_t *pos_dev, const float *table, int max_pos, llm_stream_t stream) {
+    return rope_kv_append(qkv, kc, vc, T, n_heads, n_kv_heads, head_dim, pos0, pos_dev, table, max_pos, false, stream);
+}
+
+int llm_rope_k_append(uint16_t *qkv, uint16_t *kc, uint16_t *vc, int T, int n_heads, int n_kv_heads, int head_dim,
+                      int pos0, const float *table, int max_pos, llm_stream_t stream) {
+    return rope_kv_append(qkv, kc, vc, T, n_heads, n_kv_heads, head_dim, pos0, nullptr, table, max_pos, true, stream);
 }
 
 } // extern "C"

@@ -120,6 +120,23 @@ def rope_kv_append(qkv, n_heads, n_kv_heads, head_dim, pos0, max_pos, theta=5000
     return d_q.download(), d_k.download(), d_v.download()
 
 
+def rope_k_append_attn_prefill(qkv, n_heads, n_kv_heads, head_dim, pos0, max_pos, theta=500000.0, kc=None, vc=None):
+    """The prompt pass's attention step with the queries rotated inside the attention kernel: K rotated into the
+    cache, V stored, then llm_attn_prefill_rope_q on the queries as they are.  Returns (out [T, Hq*hd], qkv
+    afterwards, K cache, V cache)."""
+    qkv = _u16(qkv)
+    T = qkv.shape[0]
+    kc = np.zeros((n_kv_heads, max_pos, head_dim), np.uint16) if kc is None else _u16(kc)
+    vc = np.zeros((n_kv_heads, head_dim, max_pos), np.uint16) if vc is None else _u16(vc)
+    d_q, d_k, d_v = DevBuf.from_host(qkv), DevBuf.from_host(kc), DevBuf.from_host(vc)
+    d_t = DevBuf.from_host(rope_table(max_pos, head_dim, theta))
+    d_o = DevBuf((T, n_heads * head_dim), np.uint16)
+    check(lib().llm_rope_k_append(d_q.ptr, d_k.ptr, d_v.ptr, T, n_heads, n_kv_heads, head_dim, pos0, d_t.ptr, max_pos, None))
+    check(lib().llm_attn_prefill_rope_q(d_q.ptr, qkv.shape[1], d_k.ptr, d_v.ptr, d_o.ptr, n_heads * head_dim, T, pos0, d_t.ptr,
+                                        n_heads, n_kv_heads, head_dim, max_pos, None))
+    return d_o.download(), d_q.download(), d_k.download(), d_v.download()
+
+
 def attn_decode(q, kc, vc, ctx, n_heads, n_kv_heads, head_dim, repeats=1):
     q, kc, vc = _u16(q), _u16(kc), _u16(vc)
     max_pos = kc.shape[1]

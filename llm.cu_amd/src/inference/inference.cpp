@@ -260,10 +260,19 @@ void issue_pass(Engine *e, const Llama3 *m, int T, int pos0, bool dev_pos, bool 
                 llama3_check(llm_linear(e->xn, d, w.wk, nullptr, 0, e->qkv + qd, QKV, T, kvd, d, s), "llm_linear(k)");
                 llama3_check(llm_linear(e->xn, d, w.wv, nullptr, 0, e->qkv + qd + kvd, QKV, T, kvd, d, s), "llm_linear(v)");
             }
-            llama3_check(llm_rope_kv_append(e->qkv, kc, vc, T, Hq, Hkv, hd, p0, pd, e->rope_table, c.max_pos, s),
-                         "llm_rope_kv_append");
-            llama3_check(llm_attn_prefill(e->qkv, QKV, kc, vc, e->attn, qd, T, p0, Hq, Hkv, hd, c.max_pos, s),
-                         "llm_attn_prefill");
+            if (!pd && T >= 16 && llm_attn_prefill_rope_q_supported(T, Hq, Hkv, hd, c.max_pos)) {
+                // the attention rotates the queries it loads: no pass over Q in memory
+                llama3_check(llm_rope_k_append(e->qkv, kc, vc, T, Hq, Hkv, hd, p0, e->rope_table, c.max_pos, s),
+                             "llm_rope_k_append");
+                llama3_check(llm_attn_prefill_rope_q(e->qkv, QKV, kc, vc, e->attn, qd, T, p0, e->rope_table, Hq, Hkv, hd,
+                                                     c.max_pos, s),
+                             "llm_attn_prefill_rope_q");
+            } else {
+                llama3_check(llm_rope_kv_append(e->qkv, kc, vc, T, Hq, Hkv, hd, p0, pd, e->rope_table, c.max_pos, s),
+                             "llm_rope_kv_append");
+                llama3_check(llm_attn_prefill(e->qkv, QKV, kc, vc, e->attn, qd, T, p0, Hq, Hkv, hd, c.max_pos, s),
+                             "llm_attn_prefill");
+            }
             llama3_check(llm_linear(e->attn, qd, w.wo, e->x, d, e->x, d, T, d, qd, s), "llm_linear(o)");
             llama3_check(llm_rmsnorm(e->x, w.post_ln, e->xn, T, d, c.rms_eps, s), "llm_rmsnorm");
             llama3_check(llm_linear_swiglu(e->xn, d, w.wg, w.wu, e->ffn, F, T, F, d, s), "llm_linear_swiglu");

@@ -467,6 +467,32 @@ def test_attn_decode_small_heads_and_gqa_map(gpu):
         assert np.allclose(got[h], h // 4 + 1, atol=2e-3)
 
 
+@pytest.mark.parametrize("T,pos0,max_pos,Hkv", [(64, 0, 128, 2), (200, 0, 256, 8), (130, 70, 256, 1), (1000, 24, 1024, 2)])
+def test_attn_prefill_that_rotates_its_queries_equals_rope_then_attention(gpu, T, pos0, max_pos, Hkv):
+    """llm_rope_k_append + llm_attn_prefill_rope_q (K rotated into the cache, V stored, the queries rotated inside
+    the attention kernel as it loads them) against llm_rope_kv_append + llm_attn_prefill: same attention output and
+    same caches bit for bit, the queries in the projection buffer left as they were, ragged last blocks and a
+    prompt appended behind cached positions included; the oracle bounds the result."""
+    hd, Hq = 128, 4 * Hkv
+    rng = np.random.default_rng(T + pos0)
+    qkv = H.bits(rng.standard_normal((T, (Hq + 2 * Hkv) * hd)))
+    kc0 = np.zeros((Hkv, max_pos, hd), np.uint16)
+    vc0 = np.zeros((Hkv, hd, max_pos), np.uint16)
+    if pos0:
+        kc0[:, :pos0] = H.bits(rng.standard_normal((Hkv, pos0, hd)))
+        vc0[:, :, :pos0] = H.bits(rng.standard_normal((Hkv, hd, pos0)))
+    say("attn prefill with its own rope", T, pos0, max_pos, Hkv)
+    assert gpu.lib().llm_attn_prefill_rope_q_supported(T, Hq, Hkv, hd, max_pos) == 1
+    q_rot, kc_r, vc_r = gpu.ops.rope_kv_append(qkv, Hq, Hkv, hd, pos0, max_pos, kc=kc0, vc=vc0)
+    want = gpu.ops.attn_prefill(q_rot[:, :Hq * hd].copy(), kc_r, vc_r, pos0, Hq, Hkv, hd)
+    got, qkv_after, kc_f, vc_f = gpu.ops.rope_k_append_attn_prefill(qkv, Hq, Hkv, hd, pos0, max_pos, kc=kc0, vc=vc0)
+    assert np.array_equal(kc_f, kc_r) and np.array_equal(vc_f, vc_r)
+    assert np.array_equal(qkv_after, qkv)
+    assert np.array_equal(got, want)
+    assert gpu.lib().llm_attn_prefill_rope_q_supported(63, Hq, Hkv, hd, max_pos) == 0
+    assert gpu.lib().llm_attn_prefill_rope_q_supported(T, 8 * Hkv, Hkv, hd, max_pos) == 0
+
+
 @pytest.mark.parametrize("T,pos0,Hq,Hkv,hd", [(1, 0, 8, 2, 32), (16, 0, 8, 2, 32), (33, 7, 8, 2, 32),
                                               (64, 0, 32, 8, 128), (100, 60, 32, 8, 128), (512, 0, 32, 8, 128),
                                               # fewer than 64 rows at the 8B head shape: the kernel of the short blocks
