@@ -100,6 +100,11 @@ struct Engine {
 };
 
 const int LONG_ATTN_FROM = 512; // cached positions from which the span + merge attention is faster
+// Prompt passes of this many rows and more leave the rotation of the queries to the attention kernel (one pass over Q
+// in memory less: 134 MB per layer at 8192 rows); below, the rotation in the attention's prologue (its first tile loads
+// wait for queries and angles, about 4 us per launch) costs more than the smaller RoPE launch saves (5 us at any size
+// up to a thousand rows).  Same bits either way.
+constexpr int ROPE_IN_ATTENTION_FROM = 4096;
 
 Engine *eng(const CudaCache *c) {
     if (!c || !c->engine) llama3_fail("CudaCache was not created by init_cache");
@@ -260,7 +265,7 @@ void issue_pass(Engine *e, const Llama3 *m, int T, int pos0, bool dev_pos, bool 
                 llama3_check(llm_linear(e->xn, d, w.wk, nullptr, 0, e->qkv + qd, QKV, T, kvd, d, s), "llm_linear(k)");
                 llama3_check(llm_linear(e->xn, d, w.wv, nullptr, 0, e->qkv + qd + kvd, QKV, T, kvd, d, s), "llm_linear(v)");
             }
-            if (!pd && T >= 16 && llm_attn_prefill_rope_q_supported(T, Hq, Hkv, hd, c.max_pos)) {
+            if (!pd && T >= ROPE_IN_ATTENTION_FROM && llm_attn_prefill_rope_q_supported(T, Hq, Hkv, hd, c.max_pos)) {
                 // the attention rotates the queries it loads: no pass over Q in memory
                 llama3_check(llm_rope_k_append(e->qkv, kc, vc, T, Hq, Hkv, hd, p0, e->rope_table, c.max_pos, s),
                              "llm_rope_k_append");
