@@ -82,6 +82,7 @@ def main():
     ap.add_argument("--cpu-steps", type=int, default=8)
     ap.add_argument("--no-graph", action="store_true")
     ap.add_argument("--no-batch", action="store_true")
+    ap.add_argument("--batch-sizes", default="4,16", help="batch sizes of the batched-decode leg (comma separated, 2..16)")
     ap.add_argument("--no-api-loop", action="store_true",
                     help="skip the three inference()-per-token legs (counter runs: thousands of launches less)")
     ap.add_argument("--no-decode-8k", action="store_true", help="skip the 64 decode steps behind the 8192-token prompt")
@@ -185,8 +186,8 @@ def main():
     if not a.no_batch:
         batched = {}
         bcfg = eng_mod.config("8b", max_pos=512)
-        for B in (4, 16):
-            engines = [eng_mod.Engine(model, bcfg) for _ in range(B)]
+        for B in [int(v) for v in a.batch_sizes.split(",") if v]:
+            engines = [eng_mod.Engine(model, bcfg, use_graph=not a.no_graph) for _ in range(B)]
             cur = []
             for b, e in enumerate(engines):
                 t, _ = e.prefill(eng_mod.seeded_tokens(a.seed + 10 + b, a.prompt, bcfg.vocab))
